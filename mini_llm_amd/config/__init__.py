@@ -2,6 +2,7 @@ from .base import ConfigError, ModelConfig, read_config_json
 from .gimozen import GimozenConfig
 from .gpt2 import GPT2Config
 from .ketolix import KetolixConfig
+from .perezen import PerezenConfig
 from .registry import (
     Architecture,
     architecture_name,
@@ -19,6 +20,7 @@ __all__ = [
     "GPT2Config",
     "KetolixConfig",
     "ModelConfig",
+    "PerezenConfig",
     "architecture_name",
     "config_from_dict",
     "get_architecture",

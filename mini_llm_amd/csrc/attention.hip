@@ -3,7 +3,7 @@
 // Pages of one cache layer: [num_pages, n_kv_heads, page_size, head_size], so the rows of one
 // head inside a page lie together. A request's block table names its pages in order. A token at
 // position p attends to the cached keys max(0, p - window + 1) .. p of its request (window 0 =
-// all), which after cache_write include the tokens of its own step: decoding and prompt
+// all; or, with chunks, to the keys of its own chunk up to p), which after cache_write include the tokens of its own step: decoding and prompt
 // portions are the same kernel.
 #include "common.h"
 #include "key_sweep.h"
@@ -37,10 +37,19 @@ constexpr int MAX_HEAD = 256;
 // (online softmax, as the reference's prefill kernel does: engine/src/attention.cu:71-124).
 // What a mixer may ask of the scores beyond scale, mask and softmax. softcap > 0: score <- softcap tanh(score / softcap),
 // behind the scale. sinks [n_heads]: exp(sink_h) joins the softmax's denominator of head h, once, with no key and no value.
+// chunk > 0: the sequence is cut into chunks of so many positions, counted from position 0, and a query sees only the keys of its own
+// chunk (up to itself): its first key is the chunk's start instead of a window's.
 struct ScoreOptions {
     float softcap;
     const float* sinks;
+    int chunk;
 };
+
+// The first key a query at `position` sees: the start of its chunk, or of its window, or key 0. It never falls as the position grows.
+__device__ __forceinline__ int first_visible_key(int position, int window, int chunk) {
+    if (chunk > 0) return position - position % chunk;
+    return window > 0 ? max(0, position - window + 1) : 0;
+}
 
 // cap tanh(s / cap). EXACT: the library's tanhf; else 1 - 2 / (1 + e^(2x)) with the hardware's 2^x and reciprocal, for
 // scores that meet bfloat16 keys.
@@ -71,7 +80,7 @@ __global__ __launch_bounds__(256) void attention_general_kernel(
     }
     const int kv_head = head / (n_heads / n_kv_heads);
     const int position = positions[token];
-    const int first_key = window > 0 ? max(0, position - window + 1) : 0;
+    const int first_key = first_visible_key(position, window, options.chunk);
     const int* table = block_tables + (size_t)request * max_blocks;
 
     float* my_q = q_shared[wave];
@@ -156,14 +165,14 @@ MLLM_API int mllm_attention(const void* q, int q_stride, const void* k_pages, co
                             void* out, int out_stride, const int* token_request,
                             const int* positions, const int* block_tables, int max_blocks,
                             int n_tokens, int n_heads, int n_kv_heads, int head_size, int page_size,
-                            int window, float scale, int dtype, float softcap, const float* sinks, hipStream_t stream) {
+                            int window, float scale, int dtype, float softcap, const float* sinks, int chunk, hipStream_t stream) {
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention: bad sizes");
-    const ScoreOptions options = {softcap, sinks};
+    const ScoreOptions options = {softcap, sinks, chunk};
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention: %d heads do not divide into %d key/value heads",
                  n_heads, n_kv_heads);
     MLLM_REQUIRE(head_size > 0 && head_size <= MAX_HEAD,
                  "attention: head size %d is not in 1..%d", head_size, MAX_HEAD);
-    MLLM_REQUIRE(page_size > 0 && window >= 0, "attention: bad page size or window");
+    MLLM_REQUIRE(page_size > 0 && window >= 0 && chunk >= 0, "attention: bad page size, window or chunk");
     MLLM_REQUIRE(q_stride >= n_heads * head_size && out_stride >= n_heads * head_size,
                  "attention: rows are too short for the heads");
     if (n_tokens == 0) return 0;
@@ -233,7 +242,7 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     }
     const int position = positions[token];
     constexpr int KPI = KeySweep<T, HD>::KPI;
-    int first_key = window > 0 ? max(0, position - window + 1) : 0;
+    int first_key = first_visible_key(position, window, options.chunk);
     int last_key = position + 1;  // exclusive
     if (n_parts > 1) {  // this block's run of the keys, in whole rounds of the sweep
         const int run = (((last_key - first_key + n_parts - 1) / n_parts + KPI - 1) / KPI) * KPI;
@@ -374,7 +383,8 @@ int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pa
     // order is 5 % faster.
     const int reach = max_blocks << page_shift;
     const int keys_per_round = (sizeof(T) == 2 ? 4096 : 2048) / head_size;  // KeySweep's KPI
-    const int rounds = ceil_div(ceil_div(window > 0 && window < reach ? window : reach, n_splits * n_parts), keys_per_round);
+    const int seen = options.chunk > 0 ? options.chunk : window;   // the most keys a token sees, if a mask bounds them
+    const int rounds = ceil_div(ceil_div(seen > 0 && seen < reach ? seen : reach, n_splits * n_parts), keys_per_round);
     const bool together = sizeof(T) == 2 || rounds <= 12;
 #define MLLM_DECODE_CASE(HD)                                                                                   \
     case HD:                                                                                                   \
@@ -413,13 +423,13 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
                                    const int* block_tables, int max_blocks, int n_tokens, int n_heads,
                                    int n_kv_heads, int head_size, int page_size, int window, float scale,
                                    int n_splits, int dtype, int out_packed, int n_parts, float* parts, int* arrivals,
-                                   float softcap, const float* sinks, hipStream_t stream) {
-    const ScoreOptions options = {softcap, sinks};
+                                   float softcap, const float* sinks, int chunk, hipStream_t stream) {
+    const ScoreOptions options = {softcap, sinks, chunk};
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_decode: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_decode: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(mllm_attention_decode_supported(head_size, page_size, dtype),
                  "attention_decode: head size %d is not one of 16, 32, 64, 128, 256, or page size %d is no power of two", head_size, page_size);
-    MLLM_REQUIRE(window >= 0, "attention_decode: bad window");
+    MLLM_REQUIRE(window >= 0 && chunk >= 0, "attention_decode: bad window or chunk");
     MLLM_REQUIRE(n_splits >= 1 && n_splits <= DECODE_MAX_SPLITS && (n_splits & (n_splits - 1)) == 0,
                  "attention_decode: %d splits is not a power of two in 1..%d", n_splits, DECODE_MAX_SPLITS);
     MLLM_REQUIRE(q_stride >= n_heads * head_size && out_stride >= n_heads * head_size, "attention_decode: rows are too short for the heads");
@@ -545,7 +555,8 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
     float running_max = -INFINITY, running_sum = 0.0f;
 
     const int block_last_position = context + min(tile_q0 + 32 * QG, q_len) - 1;
-    const int block_first_key = window > 0 ? max(0, context + tile_q0 - window + 1) : 0;
+    const int block_first_key = first_visible_key(context + tile_q0, window, options.chunk);
+    const bool masked_from = window > 0 || options.chunk > 0;   // the queries' first keys are not key 0
     // the pages this block walks, copied to LDS once: a tile's loads then do not wait for a lookup in memory
     const int first_page = block_first_key >> page_shift, last_page = block_last_position >> page_shift;
     const bool table_in_lds = last_page - first_page < PF_TABLE;
@@ -629,7 +640,7 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
         const int k0 = k_base + key_split * PF_KEYS;
         // a wave whose queries all lie before its tile, or whose windows have all passed it, has nothing to add
         if (!wave_active || k0 > wave_last_position) continue;
-        if (window > 0 && k0 + PF_KEYS - 1 < wave_first_position - window + 1) continue;
+        if (masked_from && k0 + PF_KEYS - 1 < first_visible_key(wave_first_position, window, options.chunk)) continue;
 
         // ---- S^T = K . Q^T : two 32-key tiles ----
         f32x16 s_acc[2];
@@ -653,7 +664,7 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
         }
         // ---- scale, mask (only where the tile touches the diagonal, a window or the tile's end), maximum ----
         float tile_max = -INFINITY;
-        const bool interior = wave_full && window == 0 && k0 + PF_KEYS - 1 <= wave_first_position;
+        const bool interior = wave_full && !masked_from && k0 + PF_KEYS - 1 <= wave_first_position;
         if (interior) {
 #pragma unroll
             for (int j = 0; j < 2; j++)
@@ -663,7 +674,7 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
                     tile_max = fmaxf(tile_max, s_acc[j][v]);
                 }
         } else {
-            const int first_allowed = window > 0 ? q_position - window + 1 : 0;
+            const int first_allowed = first_visible_key(q_position, window, options.chunk);
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -826,15 +837,15 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
                                     int out_stride, const int* q_starts, const int* context_lens,
                                     const int* block_tables, int max_blocks, int n_requests, int max_q_len,
                                     int max_len, int n_heads, int n_kv_heads, int head_size, int page_size, int window,
-                                    float scale, int dtype, float softcap, const float* sinks, hipStream_t stream) {
-    const ScoreOptions options = {softcap, sinks};
+                                    float scale, int dtype, float softcap, const float* sinks, int chunk, hipStream_t stream) {
+    const ScoreOptions options = {softcap, sinks, chunk};
     // max_len: the longest sequence after this step, or a bound on it (0 or less: what the block tables can hold); it only
     // decides how many waves share a block's keys
     MLLM_REQUIRE(n_requests >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_prefill: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_prefill: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(mllm_attention_prefill_supported(head_size, page_size),
                  "attention_prefill: head size %d is not a multiple of 16 in 16..128, or page size %d is no power of two", head_size, page_size);
-    MLLM_REQUIRE(window >= 0, "attention_prefill: bad window");
+    MLLM_REQUIRE(window >= 0 && chunk >= 0, "attention_prefill: bad window or chunk");
     MLLM_REQUIRE(q_stride >= n_heads * head_size && out_stride >= n_heads * head_size, "attention_prefill: rows are too short for the heads");
     MLLM_REQUIRE(n_requests <= 65535 && n_heads <= 65535, "attention_prefill: too many requests or heads for one launch");
     if (n_requests == 0 || max_q_len == 0) return 0;

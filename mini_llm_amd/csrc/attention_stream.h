@@ -205,7 +205,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4)
     }
 
     const int block_last_position = context + min(tile_q0 + QUERIES, q_len) - 1;
-    const int block_first_key = window > 0 ? max(0, context + tile_q0 - window + 1) : 0;
+    const int block_first_key = first_visible_key(context + tile_q0, window, options.chunk);
     const int first_base = (block_first_key / KEYS) * KEYS;
     const int n_tiles = (block_last_position - first_base) / KEYS + 1;
     const int n_mine = n_tiles > wave ? (n_tiles - wave + SPLITS - 1) / SPLITS : 0;  // tiles wave, wave + SPLITS, ...
@@ -330,7 +330,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4)
         // ---- mask (only where the tile touches the diagonal, a window or the portion's end), maximum, exponentials ----
         auto softmax = [&](int qs) {
             const int sub_first_position = context + tile_q0 + qs * 32;
-            const bool interior = window == 0 && tile_q0 + qs * 32 + 31 < q_len && k0 + KEYS - 1 <= sub_first_position;
+            const bool interior = window == 0 && options.chunk == 0 && tile_q0 + qs * 32 + 31 < q_len && k0 + KEYS - 1 <= sub_first_position;
             float tile_max = -INFINITY;
             if (options.softcap > 0.0f) {   // a capped score, left divided by the scale as the plain ones are: cap tanh(scale s / cap) / scale
                 const float back = options.softcap / scale, into = scale / options.softcap;
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4)
 #pragma unroll
                 for (int v = 0; v < 16; v++) tile_max = fmaxf(tile_max, s_acc[qs][v]);
             } else {
-                const int first_allowed = window > 0 ? q_position[qs] - window + 1 : 0;
+                const int first_allowed = q_position[qs] < 0 ? 0 : first_visible_key(q_position[qs], window, options.chunk);
                 const int key0 = k0 + 4 * half;
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
@@ -558,7 +558,7 @@ void launch(const void* q, int q_stride, const void* k_pages, const void* v_page
         // unit of its own at once (eight waves' tiles leave room for one block a unit): a long context with few queries.
         // Measured, heads of 64: 512 queries on 7,680 cached keys 38.2 against 46.7 us with four waves; but two prompts of 1,024
         // tokens (384 blocks: a second round) 19.1 against 15.9 us, one of 4,096 64.8 against 57 us.
-        const int reach = window > 0 ? min(max_len, window + 64) : max_len;
+        const int reach = options.chunk > 0 ? min(max_len, options.chunk + 64) : (window > 0 ? min(max_len, window + 64) : max_len);
         const long blocks = (long)n_heads * n_requests * ceil_div(max_q_len, wide ? 64 : 32);
         bool eight = false;
         if constexpr (HD * sizeof(T) <= 128) {  // (eight waves' tiles of rows of 256 bytes do not fit a compute unit's LDS)

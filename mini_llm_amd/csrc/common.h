@@ -68,7 +68,8 @@ enum MllmKernel : int {
     MLLM_K_DECODE_MLP_HALF, MLLM_K_PENDING_SUM, MLLM_K_PENDING_LAYERNORM, MLLM_K_GEMM_SKINNY, MLLM_K_GEMM_TILED, MLLM_K_GEMM_STREAM,
     MLLM_K_STATIC_SUM, MLLM_K_PROBE, MLLM_K_SAMPLE, MLLM_K_GEMM_BEST, MLLM_K_CHOOSE, MLLM_K_RMS_NORM, MLLM_K_HEAD_NORM,
     MLLM_K_LATENT_ROWS, MLLM_K_SILU_MUL, MLLM_K_HEADS_LINEAR, MLLM_K_LATENT_ATTENTION, MLLM_K_LATENT_MERGE, MLLM_K_PROJECTION_ROWS,
-    MLLM_K_HEAD_GATE, MLLM_K_GATED_NORM, MLLM_K_SHORT_CONV, MLLM_K_RECURRENCE, MLLM_K_KINDS
+    MLLM_K_HEAD_GATE, MLLM_K_GATED_NORM, MLLM_K_SHORT_CONV, MLLM_K_RECURRENCE, MLLM_K_MAP_ROWS,
+    MLLM_K_MAP_DIFFERENCE, MLLM_K_KINDS
 };
 void mllm_count_kernel(MllmKernel kind);
 

@@ -1,0 +1,178 @@
+// The row-wise work of attention whose heads hold several maps: each (head, map) has a query and a key of its own, all maps of a
+// head attend over the head's one value, and the maps' results are combined afterwards (differential attention subtracts the
+// second map from the first).
+//
+// The paged attention kernels know nothing of maps: they see n_heads * maps query heads over n_kv_heads * maps key/value heads.
+// With R = n_heads / n_kv_heads query heads to a key/value head, query head h = g R + r and map m are laid out as attention head
+// (g * maps + m) * R + r, so that the kernels' grouping (attention head a reads key/value head a / R) hands every query its own
+// map's keys, g * maps + m; the value head of g is stored under each of its maps' key heads.
+#include "common.h"
+
+namespace {
+
+constexpr int MAP_WAVES = 4;   // waves (items) a block
+
+// u, v -> the pair turned by position x frequency: the angle a 64-bit product brought into -pi .. pi (a 32-bit product of a position
+// in the thousands is good to 1e-4 only), its sine and cosine taken in 32-bit.
+__device__ __forceinline__ void turned(float u, float v, int position, double frequency, float& a, float& b) {
+    const double angle = (double)position * frequency;
+    const double turns = rint(angle * 0.15915494309189535);
+    float s, c;
+    sincosf((float)(angle - turns * 6.283185307179586), &s, &c);
+    a = u * c - v * s;
+    b = v * c + u * s;
+}
+
+// A wave per (row, item); a row's items are its n_heads * maps queries, then (where the layer keeps keys and values of its own: k_at
+// >= 0) its n_kv_heads * maps keys and its n_kv_heads values. `rows` are the 32-bit sums of the product that made them, [.. | q | k |
+// v | ..] at columns q_at, k_at, v_at: q as [n_heads, maps, dim], k as [n_kv_heads, maps, dim], v as [n_kv_heads, vdim].
+// A query or key: RMS norm over its dim elements (gain [dim], shared by all heads and maps; null: no norm), then of its first
+// rot_dims elements i and i + rot_dims / 2 turned as a pair by position x frequencies[i]. Queries go to q_out [row, n_kv_heads, maps, R,
+// head_size], keys to head g * maps + m of the row's slot in k_pages, a value to heads g * maps + 0 .. maps - 1 of v_pages, zeros
+// beyond dim / vdim up to head_size. Padding rows (slot < 0) store nothing.
+template <typename T>
+__global__ __launch_bounds__(64 * MAP_WAVES) void map_rows_kernel(
+    const float* __restrict__ rows, int stride, int q_at, int k_at, int v_at, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
+    float eps, const double* __restrict__ frequencies, int rot_dims, const int* __restrict__ positions, const int* __restrict__ slots,
+    T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages, int n_rows, int n_heads, int n_kv_heads, int maps, int dim,
+    int vdim, int head_size, int page_size) {
+    const int lane = threadIdx.x % WAVE;
+    const int n_q = n_heads * maps, n_k = k_at >= 0 ? n_kv_heads * maps : 0, n_v = k_at >= 0 ? n_kv_heads : 0;
+    const int per_row = n_q + n_k + n_v;
+    const long long item = (long long)blockIdx.x * MAP_WAVES + threadIdx.x / WAVE;
+    if (item >= (long long)n_rows * per_row) return;
+    const int row = (int)(item / per_row), which = (int)(item % per_row);
+    const float* in_row = rows + (size_t)row * stride;
+    const int per_group = n_heads / n_kv_heads;
+    if (which >= n_q + n_k) {   // a value head, as it is, under each of its maps
+        const int slot = slots[row];
+        if (slot < 0) return;
+        const int g = which - n_q - n_k;
+        const float* in = in_row + v_at + (size_t)g * vdim;
+        for (int m = 0; m < maps; m++) {
+            T* out = v_pages + (((size_t)(slot / page_size) * (n_kv_heads * maps) + g * maps + m) * page_size + slot % page_size) * head_size;
+            for (int d = lane; d < head_size; d += WAVE) out[d] = from_float<T>(d < vdim ? in[d] : 0.0f);
+        }
+        return;
+    }
+    const bool is_q = which < n_q;
+    const int index = is_q ? which : which - n_q;          // (head, map) as stored: head * maps + map
+    const int head = index / maps, map = index % maps;
+    const float* in = in_row + (is_q ? q_at : k_at) + (size_t)index * dim;
+    const float* gain = is_q ? q_gain : k_gain;
+    T* out;
+    if (is_q) {
+        const int g = head / per_group, r = head % per_group;
+        out = q_out + ((size_t)row * n_q + (size_t)(g * maps + map) * per_group + r) * head_size;
+    } else {
+        const int slot = slots[row];
+        if (slot < 0) return;
+        out = k_pages + (((size_t)(slot / page_size) * n_k + head * maps + map) * page_size + slot % page_size) * head_size;
+    }
+    float factor = 1.0f;
+    if (gain) {
+        float squares = 0.0f;
+        for (int d = lane; d < dim; d += WAVE) squares += in[d] * in[d];
+        factor = 1.0f / sqrtf(wave_sum(squares) / (float)dim + eps);
+    }
+    const int position = positions[row];
+    const int half = rot_dims / 2;
+    for (int d = lane; d < head_size; d += WAVE) {
+        float value = 0.0f;
+        if (d < dim) {
+            value = in[d] * factor * (gain ? gain[d] : 1.0f);
+            if (d < rot_dims) {
+                const int other = d < half ? d + half : d - half;
+                const float partner = in[other] * factor * (gain ? gain[other] : 1.0f);
+                float a, b;
+                if (d < half) turned(value, partner, position, frequencies[d], a, b);
+                else turned(partner, value, position, frequencies[other], b, a);
+                value = a;
+            }
+        }
+        out[d] = from_float<T>(value);
+    }
+}
+
+// A wave per (row, head): with a1 and a2 the results of the head's two maps (attention heads (g * 2 + 0) * R + r and (g * 2 + 1) * R + r
+// of `maps_out`, heads of head_size of which the first vdim count), x = a1 - lambda a2, out = x / sqrt(mean(x^2) + eps) * scale *
+// sigmoid(gate) -> out [row, head * vdim ..]. gate: 32-bit rows (null: no gate), the head's vdim elements at column head * vdim.
+template <typename T>
+__global__ __launch_bounds__(64 * MAP_WAVES) void map_difference_kernel(
+    const T* __restrict__ maps_out, int maps_stride, const float* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride,
+    float lambda, float eps, float scale, int n_rows, int n_heads, int n_kv_heads, int vdim, int head_size) {
+    constexpr int REGS = 4;   // heads up to 256 elements
+    const int lane = threadIdx.x % WAVE;
+    const long long item = (long long)blockIdx.x * MAP_WAVES + threadIdx.x / WAVE;
+    if (item >= (long long)n_rows * n_heads) return;
+    const int row = (int)(item / n_heads), head = (int)(item % n_heads);
+    const int per_group = n_heads / n_kv_heads;
+    const int g = head / per_group, r = head % per_group;
+    const T* first = maps_out + (size_t)row * maps_stride + (size_t)((g * 2) * per_group + r) * head_size;
+    const T* second = first + (size_t)per_group * head_size;
+    float x[REGS], gates[REGS], squares = 0.0f;
+#pragma unroll
+    for (int e = 0; e < REGS; e++) {
+        const int d = lane + e * WAVE;
+        const bool has = d < vdim;
+        x[e] = has ? to_float(first[d]) - lambda * to_float(second[d]) : 0.0f;
+        gates[e] = has && gate ? gate[(size_t)row * gate_stride + head * vdim + d] : 0.0f;
+        squares += x[e] * x[e];
+    }
+    const float factor = scale / sqrtf(wave_sum(squares) / (float)vdim + eps);
+#pragma unroll
+    for (int e = 0; e < REGS; e++) {
+        const int d = lane + e * WAVE;
+        if (d < vdim) out[(size_t)row * out_stride + head * vdim + d] = from_float<T>(x[e] * factor * (gate ? 1.0f / (1.0f + expf(-gates[e])) : 1.0f));
+    }
+}
+
+}  // namespace
+
+MLLM_API int mllm_map_rows(const float* rows, int stride, int q_at, int k_at, int v_at, const float* q_gain, const float* k_gain, float eps,
+                           const double* frequencies, int rot_dims, const int* positions, const int* slots, void* q_out, void* k_pages,
+                           void* v_pages, int n_rows, int n_heads, int n_kv_heads, int maps, int dim, int vdim, int head_size, int page_size,
+                           int dtype, hipStream_t stream) {
+    MLLM_REQUIRE(n_rows >= 0 && n_heads > 0 && n_kv_heads > 0 && maps > 0 && dim > 0 && vdim > 0 && page_size > 0, "map_rows: bad sizes");
+    MLLM_REQUIRE(n_heads % n_kv_heads == 0, "map_rows: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
+    MLLM_REQUIRE(head_size >= dim && head_size >= vdim, "map_rows: heads of %d do not hold %d / %d elements", head_size, dim, vdim);
+    MLLM_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dim, "map_rows: %d rotated elements of %d", rot_dims, dim);
+    MLLM_REQUIRE(rows != nullptr && q_out != nullptr && positions != nullptr && (rot_dims == 0 || frequencies != nullptr), "map_rows: a missing operand");
+    MLLM_REQUIRE(q_at >= 0 && q_at + n_heads * maps * dim <= stride, "map_rows: the queries lie beyond the rows");
+    MLLM_REQUIRE(k_at < 0 || (v_at >= 0 && k_at + n_kv_heads * maps * dim <= stride && v_at + n_kv_heads * vdim <= stride && slots != nullptr &&
+                              k_pages != nullptr && v_pages != nullptr),
+                 "map_rows: keys and values to keep need their columns, slots and pages");
+    if (n_rows == 0) return 0;
+    const long long items = (long long)n_rows * (n_heads * maps + (k_at >= 0 ? n_kv_heads * (maps + 1) : 0));
+    const int blocks = (int)((items + MAP_WAVES - 1) / MAP_WAVES);
+    mllm_count_kernel(MLLM_K_MAP_ROWS);
+#define MAP_ROWS_ARGS(T) rows, stride, q_at, k_at, v_at, q_gain, k_gain, eps, frequencies, rot_dims, positions, slots, (T*)q_out, (T*)k_pages, \
+                         (T*)v_pages, n_rows, n_heads, n_kv_heads, maps, dim, vdim, head_size, page_size
+    if (dtype == MLLM_F32) map_rows_kernel<float><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_ROWS_ARGS(float));
+    else if (dtype == MLLM_BF16) map_rows_kernel<bf16_t><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_ROWS_ARGS(bf16_t));
+    else MLLM_REQUIRE(false, "map_rows: unknown dtype %d", dtype);
+#undef MAP_ROWS_ARGS
+    return mllm_check_launch("map_rows");
+}
+
+MLLM_API int mllm_map_difference(const void* maps_out, int maps_stride, const float* gate, int gate_stride, void* out, int out_stride, float lambda,
+                                 float eps, float scale, int n_rows, int n_heads, int n_kv_heads, int vdim, int head_size, int dtype,
+                                 hipStream_t stream) {
+    MLLM_REQUIRE(n_rows >= 0 && n_heads > 0 && n_kv_heads > 0 && vdim > 0, "map_difference: bad sizes");
+    MLLM_REQUIRE(n_heads % n_kv_heads == 0, "map_difference: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
+    MLLM_REQUIRE(vdim <= head_size && vdim <= 256, "map_difference: heads of %d values (the kernel takes 256, the maps hold %d)", vdim, head_size);
+    MLLM_REQUIRE(maps_stride >= 2 * n_heads * head_size && out_stride >= n_heads * vdim && (gate == nullptr || gate_stride >= n_heads * vdim),
+                 "map_difference: rows are too short for the heads");
+    MLLM_REQUIRE(maps_out != nullptr && out != nullptr, "map_difference: a missing operand");
+    if (n_rows == 0) return 0;
+    const long long items = (long long)n_rows * n_heads;
+    const int blocks = (int)((items + MAP_WAVES - 1) / MAP_WAVES);
+    mllm_count_kernel(MLLM_K_MAP_DIFFERENCE);
+#define MAP_DIFFERENCE_ARGS(T) (const T*)maps_out, maps_stride, gate, gate_stride, (T*)out, out_stride, lambda, eps, scale, n_rows, n_heads, n_kv_heads, \
+                               vdim, head_size
+    if (dtype == MLLM_F32) map_difference_kernel<float><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_DIFFERENCE_ARGS(float));
+    else if (dtype == MLLM_BF16) map_difference_kernel<bf16_t><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_DIFFERENCE_ARGS(bf16_t));
+    else MLLM_REQUIRE(false, "map_difference: unknown dtype %d", dtype);
+#undef MAP_DIFFERENCE_ARGS
+    return mllm_check_launch("map_difference");
+}

@@ -397,8 +397,9 @@ def _arrivals(k_pages, rows: int, n_heads: int):
 
 
 def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None,
-                    short_rows=None, short_requests=None, packed_out=False, first_row=0, softcap: float = 0.0, sinks=None):
-    """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p).
+                    short_rows=None, short_requests=None, packed_out=False, first_row=0, softcap: float = 0.0, sinks=None, chunk: int = 0):
+    """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p; with ``chunk`` > 0 the keys of
+    the row's own chunk of so many positions, chunks counted from position 0: floor(p / chunk) * chunk .. p).
     ``softcap`` > 0: a scaled score s counts as softcap * tanh(s / softcap). ``sinks`` (float32 [n_heads]): exp(sink_h) joins
     the denominator of head h's softmax, once, with no key and no value.
 
@@ -438,7 +439,8 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     if sinks is not None:
         _device_tensor(sinks, "sinks", torch.float32, 1)
         _require(sinks.shape[0] == n_heads, "one sink a head")
-    softcap = float(softcap or 0.0)
+    softcap, chunk = float(softcap or 0.0), int(chunk or 0)
+    _require(chunk >= 0 and not (chunk and window), "the keys a row sees are bounded by a window or by chunks, not both")
     rows_aligned = q.data_ptr() % 16 == 0 and (q.stride(0) * q.element_size()) % 16 == 0  # 16-byte loads of q
     if (short_rows is not None and short_requests is not None and 0 < short_rows < n and max_q_len is not None
             and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None and rows_aligned
@@ -446,7 +448,7 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
             and lib.mllm_attention_prefill_supported(head_size, page_size)):
         _require(0 < short_requests < context_lens.shape[0], "short_requests does not cut the batch in two")
         common = dict(n_heads=n_heads, n_kv_heads=n_kv_heads, head_size=head_size, scale=scale, window=window, max_len=max_len, first_row=first_row,
-                      softcap=softcap, sinks=sinks)
+                      softcap=softcap, sinks=sinks, chunk=chunk)
         paged_attention(q[:short_rows], k_pages, v_pages, token_request, positions, block_tables, max_q_len=DECODE_MAX_Q_LEN,
                         q_starts=q_starts[: short_requests + 1], context_lens=context_lens[:short_requests],
                         out=out[:short_rows], **common)
@@ -460,8 +462,8 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         # waves per block as keep the launch within what is resident at once, never more than one
         # per 64 keys of reach
         reach = block_tables.shape[1] * page_size if max_len is None else max(1, min(max_len, block_tables.shape[1] * page_size))
-        if window:
-            reach = min(reach, int(window))
+        if window or chunk:
+            reach = min(reach, int(window or chunk))
         # few tokens with many keys: a token's keys in several runs, a block each, so that the blocks are about as many
         # as the chip has compute units, and a second small kernel that puts the runs together
         n_parts, units = 1, _compute_units(q.device)
@@ -483,7 +485,7 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), width if packed_out else out.stride(0),
                                         _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads,
                                         head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), int(packed_out),
-                                        n_parts, _ptr(parts), _ptr(arrivals), softcap, _ptr(sinks), _stream()))
+                                        n_parts, _ptr(parts), _ptr(arrivals), softcap, _ptr(sinks), chunk, _stream()))
         return result
     if (max_q_len is not None and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None
             and rows_aligned and lib.mllm_attention_prefill_supported(head_size, page_size)):
@@ -492,9 +494,9 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         n_requests = context_lens.shape[0]
         _require(q_starts.shape[0] == n_requests + 1, "q_starts must have one entry more than context_lens")
         _require(block_tables.shape[0] >= n_requests, "fewer block tables than requests")
-        check(lib.mllm_attention_prefill(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_starts), _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n_requests, int(max_q_len), int(max_len or 0), n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), _stream()))
+        check(lib.mllm_attention_prefill(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_starts), _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n_requests, int(max_q_len), int(max_len or 0), n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), chunk, _stream()))
         return out
-    check(lib.mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), _stream()))
+    check(lib.mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), chunk, _stream()))
     return out
 
 
@@ -1158,4 +1160,67 @@ def recurrence(q, k, v, state, q_starts, state_slots, n_heads, dim, vdim, *, gat
     check(library().mllm_recurrence(0 if gated else 1, _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(gate_in), _ptr(gate_forget),
                                     gate_in.stride(0) if gated else 0, float(cap or 0.0), _ptr(decay), float(q_scale), _ptr(state), state.stride(0), matrices,
                                     matrices + n_heads * dim, _ptr(q_starts), _ptr(state_slots), _ptr(out), out.stride(0), n_requests, n_heads, dim, vdim, _stream()))
+    return out
+
+
+# -- attention whose heads hold several maps over one value (differential attention) -----------------------------------------
+def map_rows(rows, q_at: int, k_at: int | None, v_at: int | None, q_gain, k_gain, eps, frequencies, rot_dims, positions, slots, k_pages, v_pages,
+             n_heads, n_kv_heads, maps, dim, vdim):
+    """The row-wise work between the fused projection of a mixer with ``maps`` maps a head and its attention. ``rows``: the float32
+    sums of that product, the queries [n_heads, maps, dim] at column ``q_at``, the keys [n_kv_heads, maps, dim] at ``k_at`` and the values
+    [n_kv_heads, vdim] at ``v_at`` (both None: the layer reads keys and values another layer keeps, and only its queries are made).
+    Every query and key is RMS-normed over its ``dim`` elements (gains [dim], shared by heads and maps; None: no norm), then of its
+    first ``rot_dims`` elements i and i + rot_dims / 2 are turned as a pair by position * frequencies[i] (float64; the angle is taken in
+    64-bit). Returns the queries as [rows, n_heads * maps * head_size] in the pages' type, laid out for the paged attention kernels run with
+    n_heads * maps heads over n_kv_heads * maps key/value heads: query head g R + r (R = n_heads / n_kv_heads) of map m is their head (g *
+    maps + m) * R + r. Keys go to head g * maps + m of slots[row] of the pages ([num_pages, n_kv_heads * maps, page_size, head_size]), the
+    value head g to the heads g * maps + 0 .. maps - 1 of the value pages; zeros beyond dim / vdim."""
+    num_pages, n_kv, page_size, head_size = k_pages.shape
+    _check_pages(k_pages, v_pages, n_kv_heads * maps, head_size)
+    _require(isinstance(rows, torch.Tensor) and rows.is_cuda and rows.dim() == 2 and rows.dtype == torch.float32 and rows.stride(1) == 1,
+             "the rows must be float32 GPU rows with contiguous columns")
+    n, width = rows.shape
+    keeps = k_at is not None
+    _require(keeps == (v_at is not None), "keys and values are kept together")
+    _require(0 <= q_at and q_at + n_heads * maps * dim <= width, "the queries lie beyond the rows")
+    _require(not keeps or (0 <= k_at and k_at + n_kv_heads * maps * dim <= width and 0 <= v_at and v_at + n_kv_heads * vdim <= width),
+             "keys or values lie beyond the rows")
+    _require(head_size >= dim and head_size >= vdim, "the pages' heads are too small")
+    for gain, name in ((q_gain, "q_gain"), (k_gain, "k_gain")):
+        if gain is not None:
+            _device_tensor(gain, name, torch.float32, 1)
+            _require(gain.shape[0] == dim, f"{name} does not match the heads")
+    if rot_dims:
+        _device_tensor(frequencies, "frequencies", torch.float64, 1)
+        _require(rot_dims % 2 == 0 and rot_dims <= dim and frequencies.shape[0] >= rot_dims // 2, "the rotation does not fit the heads")
+    _device_tensor(positions, "positions", torch.int32, 1)
+    _require(positions.shape[0] >= n, "fewer positions than rows")
+    if keeps:
+        _device_tensor(slots, "slots", torch.int32, 1)
+        _require(slots.shape[0] >= n, "fewer slots than rows")
+    out = torch.empty((n, n_heads * maps * head_size), dtype=k_pages.dtype, device=rows.device)
+    check(library().mllm_map_rows(_ptr(rows), rows.stride(0), int(q_at), int(k_at) if keeps else -1, int(v_at) if keeps else -1, _ptr(q_gain), _ptr(k_gain),
+                                  float(eps), _ptr(frequencies if rot_dims else None), int(rot_dims), _ptr(positions), _ptr(slots if keeps else None), _ptr(out),
+                                  _ptr(k_pages), _ptr(v_pages), n, n_heads, n_kv_heads, int(maps), dim, vdim, head_size, page_size, _code(k_pages.dtype),
+                                  _stream()))
+    return out
+
+
+def map_difference(maps_out, gate, lam: float, eps: float, n_heads, n_kv_heads, vdim, head_size, scale: float = 1.0, out=None):
+    """Two maps a head into one: with a1, a2 the results of a head's maps in ``maps_out`` ([rows, n_heads * 2 * head_size] as the paged
+    attention leaves them for the queries of ``map_rows``; the first ``vdim`` elements of a head count), x = a1 - lam * a2 and out = x /
+    sqrt(mean(x^2) + eps) * scale * sigmoid(gate), [rows, n_heads * vdim] of the maps' type, the heads in their own order. ``gate``:
+    float32 rows [rows, n_heads * vdim] (strided; None: no gate)."""
+    _require(maps_out.is_cuda and maps_out.dim() == 2 and maps_out.stride(1) == 1 and maps_out.shape[1] == 2 * n_heads * head_size,
+             "the maps' rows do not match the heads")
+    n = maps_out.shape[0]
+    if gate is not None:
+        _rows_f32(gate, "gate", n_heads * vdim)
+        _require(gate.shape[0] == n, "the gate's rows do not match")
+    if out is None:
+        out = torch.empty((n, n_heads * vdim), dtype=maps_out.dtype, device=maps_out.device)
+    _device_tensor(out, "out", maps_out.dtype, 2)
+    _require(tuple(out.shape) == (n, n_heads * vdim) and out.stride(1) == 1, "out has the wrong shape")
+    check(library().mllm_map_difference(_ptr(maps_out), maps_out.stride(0), _ptr(gate), 0 if gate is None else gate.stride(0), _ptr(out), out.stride(0),
+                                        float(lam), float(eps), float(scale), n, n_heads, n_kv_heads, vdim, head_size, _code(maps_out.dtype), _stream()))
     return out

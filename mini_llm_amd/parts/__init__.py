@@ -4,7 +4,8 @@ from .base import (
     Block, FeedForward, KVNeed, LayerContext, Mixer, Norm, Part, PositionEncoding, StateNeed,
     make_part, register_part,
 )
-from .block import BranchNormBlock, PostNormBlock, PreNormBlock
+from .block import BranchNormBlock, PostNormBlock, PreNormBlock, SandwichNormBlock
+from .differential_attention import DifferentialAttention
 from .embedding import LinearHead, TiedHead, TokenEmbedding
 from .feedforward import DenseMLP, GatedMLP
 from .latent_attention import LatentAttention
@@ -20,5 +21,5 @@ __all__ = [
     "make_part", "register_part",
     "CausalSelfAttention", "PreNormBlock", "TiedHead", "TokenEmbedding", "DenseMLP", "Linear", "LayerNorm", "LearnedPositions",
     "NormedHeadAttention", "LatentAttention", "BranchNormBlock", "ProjectionNormAttention", "DecayedLinearAttention",
-    "MatrixMemoryMixer", "ParallelMixer", "PostNormBlock", "LinearHead", "GatedMLP", "RMSNorm", "RotaryEncoding",
+    "MatrixMemoryMixer", "ParallelMixer", "PostNormBlock", "SandwichNormBlock", "DifferentialAttention", "LinearHead", "GatedMLP", "RMSNorm", "RotaryEncoding",
 ]

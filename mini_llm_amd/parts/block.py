@@ -96,6 +96,37 @@ class BranchNormBlock(Block):
         return self.norm_2.forward_onto(hidden.stream, self.feed_forward.forward(hidden.rows, None), self.compute_dtype)
 
 
+class SandwichNormBlock(Block):
+    """A norm in front of each branch and one on its output: x <- x + norm_1b(mixer(norm_1(x))), then x <- x + norm_2b(feed_forward(norm_2(x))).
+    ``feed_forward`` None: the layer ends behind its mixer. The stream is float32 rows; the norms on the outputs have ``forward_added``
+    (RMSNorm: stream + norm(branch) from one kernel, which also adds up the partial products of a branch whose last product was cut
+    along K), and mixer and feed-forward return their branch alone when given no residual."""
+
+    def __init__(self, norm_1: Norm, mixer: Mixer, norm_1b: Norm, norm_2: Norm | None, feed_forward: FeedForward | None, norm_2b: Norm | None,
+                 compute_dtype, names=("norm1", "mix.", "norm1b", "norm2", "mlp.", "norm2b")):
+        if not ((norm_2 is None) == (feed_forward is None) == (norm_2b is None)):
+            raise ValueError("the second pair of norms goes with the feed-forward")
+        self.norm_1, self.mixer, self.norm_1b, self.norm_2, self.feed_forward, self.norm_2b = norm_1, mixer, norm_1b, norm_2, feed_forward, norm_2b
+        self.compute_dtype = compute_dtype
+        self._names = names
+
+    def children(self):
+        parts = dict(zip(self._names, (self.norm_1, self.mixer, self.norm_1b, self.norm_2, self.feed_forward, self.norm_2b)))
+        return {name: part for name, part in parts.items() if part is not None}
+
+    def mixer_part(self):
+        return self.mixer
+
+    def forward(self, hidden, ctx: LayerContext):
+        branch = self.mixer.forward(self.norm_1.forward(hidden, self.compute_dtype), None, ctx)
+        hidden = self.norm_1b.forward_added(hidden, branch)
+        if self.feed_forward is None:
+            return hidden
+        branch = self.feed_forward.forward(self.norm_2.forward(hidden, self.compute_dtype), None)
+        return self.norm_2b.forward_added(hidden, branch)
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "sandwich_norm", SandwichNormBlock)
 register_part("block", "post_norm", PostNormBlock)
 register_part("block", "branch_norm", BranchNormBlock)

@@ -34,12 +34,16 @@ class LayerNorm(Norm):
 
 class RMSNorm(Norm):
     """x / sqrt(mean(x^2) + eps) * g, in 32-bit. ``one_plus``: the stored vector lies around zero and g = 1 + weight.
-    ``tensor_name``: the vector's name behind the part's prefix ("" where the part's own name is the tensor's)."""
+    ``tensor_name``: the vector's name behind the part's prefix ("" where the part's own name is the tensor's). ``out_scale``: a
+    constant that multiplies the normed rows, folded into the 32-bit gain when the weights are bound (a model whose logits are scaled
+    gives its final norm the scale: the head's product is linear)."""
 
-    def __init__(self, width: int, eps: float, one_plus: bool = False, tensor_name: str = "weight"):
+    def __init__(self, width: int, eps: float, one_plus: bool = False, tensor_name: str = "weight", out_scale: float = 1.0):
         if not eps > 0:
             raise ValueError(f"eps must be positive, not {eps}")
-        self.width, self.eps, self.one_plus = width, float(eps), bool(one_plus)
+        if out_scale != 1.0 and one_plus:
+            raise ValueError("a scale is folded into a plain gain vector, not into one stored around zero")
+        self.width, self.eps, self.one_plus, self.out_scale = width, float(eps), bool(one_plus), float(out_scale)
         self._tensor_name = tensor_name
         self.weight = None
 
@@ -48,6 +52,8 @@ class RMSNorm(Norm):
 
     def bind(self, tensors):
         self.weight = tensors[self._tensor_name]
+        if self.out_scale != 1.0:
+            self.weight = (self.weight.double() * self.out_scale).float()
 
     def forward(self, x, out_dtype, row_index=None):
         return kernels.rms_norm(x, self.weight, self.eps, one_plus=self.one_plus, out_dtype=out_dtype, row_index=row_index)
@@ -60,6 +66,14 @@ class RMSNorm(Norm):
             return kernels.NormedRows(stream, stream)
         return kernels.NormedRows(*kernels.rms_norm(x, self.weight, self.eps, addend=addend, alpha=alpha, one_plus=self.one_plus,
                                                     out_dtype=out_dtype, with_stream=True))
+
+    def forward_added(self, stream, branch):
+        """stream + norm(branch) in float32 alone: for a layer whose next branch has a norm of its own in front. ``branch`` as for
+        ``forward_onto``."""
+        addend = None
+        if branch.dim() == 3:
+            branch, addend = branch[0], (branch[1:] if branch.shape[0] > 1 else None)
+        return kernels.rms_norm(branch, self.weight, self.eps, addend=addend, one_plus=self.one_plus, residual=stream)
 
     def forward_onto(self, stream, branch, out_dtype):
         """stream + norm(branch) -> kernels.NormedRows: the sum of a layer whose norm sits on its branch's output, in float32 and in

@@ -8,14 +8,20 @@ from .base import PositionEncoding, register_part
 
 
 class LearnedPositions(PositionEncoding):
+    """``tensor_name``: the table's name behind the part's prefix ("" where the part's own name is the tensor's)."""
+
     stage = "embedding"
 
-    def __init__(self, n_positions: int, width: int):
+    def __init__(self, n_positions: int, width: int, tensor_name: str = "weight", std: float = 0.02):
         self.n_positions, self.width = n_positions, width
+        self._tensor_name, self._std = tensor_name, std
         self.weight = None
 
     def tensor_specs(self):
-        return {"weight": TensorSpec((self.n_positions, self.width), TABLE, Normal(0.02))}
+        return {self._tensor_name: TensorSpec((self.n_positions, self.width), TABLE, Normal(self._std))}
+
+    def bind(self, tensors):
+        self.weight = tensors[self._tensor_name]
 
     def max_positions(self) -> int:
         return self.n_positions
