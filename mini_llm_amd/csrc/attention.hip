@@ -39,11 +39,21 @@ constexpr int MAX_HEAD = 256;
 // behind the scale. sinks [n_heads]: exp(sink_h) joins the softmax's denominator of head h, once, with no key and no value.
 // chunk > 0: the sequence is cut into chunks of so many positions, counted from position 0, and a query sees only the keys of its own
 // chunk (up to itself): its first key is the chunk's start instead of a window's.
+// wide_out: the results leave as 32-bit floats whatever the pages' type (`out` is then a float array and `out_stride` counts floats):
+// for a mixer that goes on computing with them before anything is rounded.
 struct ScoreOptions {
     float softcap;
     const float* sinks;
     int chunk;
+    int wide_out;
 };
+
+// out[index] = value, as T or (wide) as a 32-bit float.
+template <typename T>
+__device__ __forceinline__ void store_result(T* out, size_t index, float value, bool wide) {
+    if (sizeof(T) == 4 || !wide) out[index] = from_float<T>(value);
+    else reinterpret_cast<float*>(out)[index] = value;
+}
 
 // The first key a query at `position` sees: the start of its chunk, or of its window, or key 0. It never falls as the position grows.
 __device__ __forceinline__ int first_visible_key(int position, int window, int chunk) {
@@ -73,9 +83,9 @@ __global__ __launch_bounds__(256) void attention_general_kernel(
     const int head = blockIdx.y * 4 + wave;
     if (head >= n_heads) return;  // no block-wide barrier below
     const int request = token_request[token];
-    T* out_row = out + (size_t)token * out_stride + head * head_size;
+    const size_t out_row = (size_t)token * out_stride + head * head_size;
     if (request < 0) {
-        for (int d = lane; d < head_size; d += WAVE) out_row[d] = from_float<T>(0.0f);
+        for (int d = lane; d < head_size; d += WAVE) store_result(out, out_row + d, 0.0f, options.wide_out);
         return;
     }
     const int kv_head = head / (n_heads / n_kv_heads);
@@ -132,7 +142,7 @@ __global__ __launch_bounds__(256) void attention_general_kernel(
 #pragma unroll
     for (int r = 0; r < REGS; r++) {
         int d = lane + r * WAVE;
-        if (d < head_size) out_row[d] = from_float<T>(o[r] * inverse);
+        if (d < head_size) store_result(out, out_row + d, o[r] * inverse, options.wide_out);
     }
 }
 
@@ -165,9 +175,9 @@ MLLM_API int mllm_attention(const void* q, int q_stride, const void* k_pages, co
                             void* out, int out_stride, const int* token_request,
                             const int* positions, const int* block_tables, int max_blocks,
                             int n_tokens, int n_heads, int n_kv_heads, int head_size, int page_size,
-                            int window, float scale, int dtype, float softcap, const float* sinks, int chunk, hipStream_t stream) {
+                            int window, float scale, int dtype, float softcap, const float* sinks, int chunk, int wide_out, hipStream_t stream) {
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention: bad sizes");
-    const ScoreOptions options = {softcap, sinks, chunk};
+    const ScoreOptions options = {softcap, sinks, chunk, wide_out};
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention: %d heads do not divide into %d key/value heads",
                  n_heads, n_kv_heads);
     MLLM_REQUIRE(head_size > 0 && head_size <= MAX_HEAD,
@@ -231,13 +241,14 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     const int request = token_request[token];
     // out_packed: the rows go out in the packed layout of a [tokens, n_heads * HD] matrix, for the
     // output product of few rows that reads them next
-    auto out_at = [&](int d) -> T* {
-        return out + (out_packed ? packed_element<T>(token, head * HD + d, n_heads * HD) : (size_t)token * out_stride + head * HD + d);
+    auto put_out = [&](int d, float value) {
+        store_result(out, out_packed ? packed_element<T>(token, head * HD + d, n_heads * HD) : (size_t)token * out_stride + head * HD + d, value,
+                     options.wide_out);
     };
     const int n_parts = gridDim.z, part = blockIdx.z;
     if (request < 0) {  // a padding row; the whole block leaves together (its zeros come from the block of the first run)
         if (part == 0)
-            for (int d = threadIdx.x; d < HD; d += blockDim.x) *out_at(d) = from_float<T>(0.0f);
+            for (int d = threadIdx.x; d < HD; d += blockDim.x) put_out(d, 0.0f);
         return;
     }
     const int position = positions[token];
@@ -356,7 +367,7 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
 #pragma unroll
                 for (int u = 0; u < 4; u++) value += p0 + u < n_parts ? o[u] * __shfl(factor, p0 + u, WAVE) : 0.0f;
             }
-            if (d0 + lane < HD) *out_at(d) = from_float<T>(value * one_over);
+            if (d0 + lane < HD) put_out(d, value * one_over);
         }
         return;
     }
@@ -365,7 +376,7 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     for (int d = threadIdx.x; d < HD; d += blockDim.x) {
         float value = 0.0f;
         for (int s = 0; s < n_splits; s++) value += partial[s][d] * expf(partial[s][HD] - total_max);
-        *out_at(d) = from_float<T>(value * inverse);
+        put_out(d, value * inverse);
     }
 }
 
@@ -423,8 +434,9 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
                                    const int* block_tables, int max_blocks, int n_tokens, int n_heads,
                                    int n_kv_heads, int head_size, int page_size, int window, float scale,
                                    int n_splits, int dtype, int out_packed, int n_parts, float* parts, int* arrivals,
-                                   float softcap, const float* sinks, int chunk, hipStream_t stream) {
-    const ScoreOptions options = {softcap, sinks, chunk};
+                                   float softcap, const float* sinks, int chunk, int wide_out, hipStream_t stream) {
+    const ScoreOptions options = {softcap, sinks, chunk, wide_out};
+    MLLM_REQUIRE(!(wide_out && out_packed), "attention_decode: rows in the packed layout leave in the pages' type");
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_decode: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_decode: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(mllm_attention_decode_supported(head_size, page_size, dtype),
@@ -780,13 +792,13 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
     if (!q_valid) return;
     if (options.sinks) running_sum += softmax_exp<HALF>(options.sinks[head] * (HALF ? LOG2E : 1.0f) - running_max);
     float inverse = 1.0f / running_sum;  // every query sees at least its own key
-    T* out_row = out + (size_t)(q_first + q_local) * out_stride + head * head_size;
+    const size_t out_row = (size_t)(q_first + q_local) * out_stride + head * head_size;
 #pragma unroll
     for (int i = 0; i < DT; i++)
 #pragma unroll
         for (int v = 0; v < 16; v++) {
             int d = i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
-            if (d < head_size) out_row[d] = from_float<T>(acc_o[i][v] * inverse);
+            if (d < head_size) store_result(out, out_row + d, acc_o[i][v] * inverse, options.wide_out);
         }
 }
 
@@ -837,8 +849,8 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
                                     int out_stride, const int* q_starts, const int* context_lens,
                                     const int* block_tables, int max_blocks, int n_requests, int max_q_len,
                                     int max_len, int n_heads, int n_kv_heads, int head_size, int page_size, int window,
-                                    float scale, int dtype, float softcap, const float* sinks, int chunk, hipStream_t stream) {
-    const ScoreOptions options = {softcap, sinks, chunk};
+                                    float scale, int dtype, float softcap, const float* sinks, int chunk, int wide_out, hipStream_t stream) {
+    const ScoreOptions options = {softcap, sinks, chunk, wide_out};
     // max_len: the longest sequence after this step, or a bound on it (0 or less: what the block tables can hold); it only
     // decides how many waves share a block's keys
     MLLM_REQUIRE(n_requests >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_prefill: bad sizes");
@@ -860,7 +872,8 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
 #define MLLM_STREAM_CASE(T, HD)                                                                                            \
     prefill_stream::launch<T, HD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,    \
                                   max_blocks, n_requests, max_q_len, reach, n_heads, n_kv_heads, page_shift, window, scale, options, stream)
-    if (dtype == MLLM_BF16 && prefill_stream::takes<bf16_t>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
+    if (dtype == MLLM_BF16 && (!wide_out || ((size_t)out) % 16 == 0) &&
+        prefill_stream::takes<bf16_t>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
         // long portions, rows of 64 / 128 / 256 bytes, pages of 32 keys or more: keys and values stream from the pages straight into LDS
         if (head_size == 32) MLLM_STREAM_CASE(bf16_t, 32);
         else if (head_size == 64) MLLM_STREAM_CASE(bf16_t, 64);

@@ -490,7 +490,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4)
         }
         if (options.sinks) total += weight_of(options.sinks[head] * (FP32 ? 1.0f : 1.4426950408889634f) - best);   // the sink: once, with no value
         const float inverse = 1.0f / total;
-        T* out_row = out + (size_t)(q_first + q_local) * out_stride + head * HD + i2 * 32;
+        const size_t out_row = (size_t)(q_first + q_local) * out_stride + head * HD + i2 * 32;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             float o[4];
@@ -502,8 +502,9 @@ __global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4)
                     sum += weight[w] * reinterpret_cast<const float*>(lds + w * L::WAVE_BYTES)[(share * 16 + 4 * g + e) * WAVE + lane];
                 o[e] = sum * inverse;
             }
-            if constexpr (FP32) *reinterpret_cast<f32x4*>(out_row + 8 * g + 4 * half) = f32x4{o[0], o[1], o[2], o[3]};
-            else *reinterpret_cast<bf16x4*>(out_row + 8 * g + 4 * half) = bf16x4{static_cast<bf16_t>(o[0]), static_cast<bf16_t>(o[1]), static_cast<bf16_t>(o[2]), static_cast<bf16_t>(o[3])};
+            const size_t at = out_row + 8 * g + 4 * half;
+            if (FP32 || options.wide_out) *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(out) + at) = f32x4{o[0], o[1], o[2], o[3]};
+            else *reinterpret_cast<bf16x4*>(out + at) = bf16x4{static_cast<bf16_t>(o[0]), static_cast<bf16_t>(o[1]), static_cast<bf16_t>(o[2]), static_cast<bf16_t>(o[3])};
         }
     }
 }

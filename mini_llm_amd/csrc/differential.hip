@@ -96,10 +96,11 @@ __global__ __launch_bounds__(64 * MAP_WAVES) void map_rows_kernel(
 
 // A wave per (row, head): with a1 and a2 the results of the head's two maps (attention heads (g * 2 + 0) * R + r and (g * 2 + 1) * R + r
 // of `maps_out`, heads of head_size of which the first vdim count), x = a1 - lambda a2, out = x / sqrt(mean(x^2) + eps) * scale *
-// sigmoid(gate) -> out [row, head * vdim ..]. gate: 32-bit rows (null: no gate), the head's vdim elements at column head * vdim.
-template <typename T>
+// sigmoid(gate) -> out [row, head * vdim ..]. gate: 32-bit rows (null: no gate), the head's vdim elements at column head * vdim. The
+// maps' results may be of another type than out (32-bit results of the attention, out in the type the output product reads).
+template <typename TIN, typename T>
 __global__ __launch_bounds__(64 * MAP_WAVES) void map_difference_kernel(
-    const T* __restrict__ maps_out, int maps_stride, const float* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride,
+    const TIN* __restrict__ maps_out, int maps_stride, const float* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride,
     float lambda, float eps, float scale, int n_rows, int n_heads, int n_kv_heads, int vdim, int head_size) {
     constexpr int REGS = 4;   // heads up to 256 elements
     const int lane = threadIdx.x % WAVE;
@@ -108,8 +109,8 @@ __global__ __launch_bounds__(64 * MAP_WAVES) void map_difference_kernel(
     const int row = (int)(item / n_heads), head = (int)(item % n_heads);
     const int per_group = n_heads / n_kv_heads;
     const int g = head / per_group, r = head % per_group;
-    const T* first = maps_out + (size_t)row * maps_stride + (size_t)((g * 2) * per_group + r) * head_size;
-    const T* second = first + (size_t)per_group * head_size;
+    const TIN* first = maps_out + (size_t)row * maps_stride + (size_t)((g * 2) * per_group + r) * head_size;
+    const TIN* second = first + (size_t)per_group * head_size;
     float x[REGS], gates[REGS], squares = 0.0f;
 #pragma unroll
     for (int e = 0; e < REGS; e++) {
@@ -156,7 +157,7 @@ MLLM_API int mllm_map_rows(const float* rows, int stride, int q_at, int k_at, in
 }
 
 MLLM_API int mllm_map_difference(const void* maps_out, int maps_stride, const float* gate, int gate_stride, void* out, int out_stride, float lambda,
-                                 float eps, float scale, int n_rows, int n_heads, int n_kv_heads, int vdim, int head_size, int dtype,
+                                 float eps, float scale, int n_rows, int n_heads, int n_kv_heads, int vdim, int head_size, int in_dtype, int dtype,
                                  hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && n_heads > 0 && n_kv_heads > 0 && vdim > 0, "map_difference: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "map_difference: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
@@ -168,11 +169,12 @@ MLLM_API int mllm_map_difference(const void* maps_out, int maps_stride, const fl
     const long long items = (long long)n_rows * n_heads;
     const int blocks = (int)((items + MAP_WAVES - 1) / MAP_WAVES);
     mllm_count_kernel(MLLM_K_MAP_DIFFERENCE);
-#define MAP_DIFFERENCE_ARGS(T) (const T*)maps_out, maps_stride, gate, gate_stride, (T*)out, out_stride, lambda, eps, scale, n_rows, n_heads, n_kv_heads, \
-                               vdim, head_size
-    if (dtype == MLLM_F32) map_difference_kernel<float><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_DIFFERENCE_ARGS(float));
-    else if (dtype == MLLM_BF16) map_difference_kernel<bf16_t><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_DIFFERENCE_ARGS(bf16_t));
-    else MLLM_REQUIRE(false, "map_difference: unknown dtype %d", dtype);
+#define MAP_DIFFERENCE_ARGS(TIN, T) (const TIN*)maps_out, maps_stride, gate, gate_stride, (T*)out, out_stride, lambda, eps, scale, n_rows, n_heads, \
+                                    n_kv_heads, vdim, head_size
+    if (in_dtype == MLLM_F32 && dtype == MLLM_F32) map_difference_kernel<float, float><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_DIFFERENCE_ARGS(float, float));
+    else if (in_dtype == MLLM_F32 && dtype == MLLM_BF16) map_difference_kernel<float, bf16_t><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_DIFFERENCE_ARGS(float, bf16_t));
+    else if (in_dtype == MLLM_BF16 && dtype == MLLM_BF16) map_difference_kernel<bf16_t, bf16_t><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_DIFFERENCE_ARGS(bf16_t, bf16_t));
+    else MLLM_REQUIRE(false, "map_difference: maps of dtype %d into rows of dtype %d", in_dtype, dtype);
 #undef MAP_DIFFERENCE_ARGS
     return mllm_check_launch("map_difference");
 }

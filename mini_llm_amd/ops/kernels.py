@@ -397,11 +397,12 @@ def _arrivals(k_pages, rows: int, n_heads: int):
 
 
 def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None,
-                    short_rows=None, short_requests=None, packed_out=False, first_row=0, softcap: float = 0.0, sinks=None, chunk: int = 0):
+                    short_rows=None, short_requests=None, packed_out=False, first_row=0, softcap: float = 0.0, sinks=None, chunk: int = 0, wide_out: bool = False):
     """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p; with ``chunk`` > 0 the keys of
     the row's own chunk of so many positions, chunks counted from position 0: floor(p / chunk) * chunk .. p).
     ``softcap`` > 0: a scaled score s counts as softcap * tanh(s / softcap). ``sinks`` (float32 [n_heads]): exp(sink_h) joins
-    the denominator of head h's softmax, once, with no key and no value.
+    the denominator of head h's softmax, once, with no key and no value. ``wide_out``: the result is float32 whatever the pages' type
+    is (for a mixer that goes on computing with the heads' results before anything is rounded); not together with ``packed_out``.
 
     q is a 2-D view [rows, n_heads*head_size] (rows may be strided); token_request[row] is the
     row of block_tables that holds the request's pages (negative: padding row, output zero).
@@ -429,10 +430,13 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     _device_tensor(positions, "positions", torch.int32, 1)
     _device_tensor(block_tables, "block_tables", torch.int32, 2)
     _require(token_request.shape[0] >= n and positions.shape[0] >= n, "fewer positions than rows")
+    wide_out = bool(wide_out)
+    _require(not (wide_out and packed_out), "rows in the packed layout leave in the pages' type")
+    out_dtype = torch.float32 if wide_out else q.dtype
     if out is None:
-        out = torch.empty((n, width), dtype=q.dtype, device=q.device)
-    _device_tensor(out, "out", q.dtype, 2)
-    _require(tuple(out.shape) == (n, width), "out has the wrong shape")
+        out = torch.empty((n, width), dtype=out_dtype, device=q.device)
+    _device_tensor(out, "out", out_dtype, 2)
+    _require(tuple(out.shape) == (n, width) and out.stride(1) == 1, "out has the wrong shape")
     lib = library()
     if n == 0:
         return out
@@ -448,7 +452,7 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
             and lib.mllm_attention_prefill_supported(head_size, page_size)):
         _require(0 < short_requests < context_lens.shape[0], "short_requests does not cut the batch in two")
         common = dict(n_heads=n_heads, n_kv_heads=n_kv_heads, head_size=head_size, scale=scale, window=window, max_len=max_len, first_row=first_row,
-                      softcap=softcap, sinks=sinks, chunk=chunk)
+                      softcap=softcap, sinks=sinks, chunk=chunk, wide_out=wide_out)
         paged_attention(q[:short_rows], k_pages, v_pages, token_request, positions, block_tables, max_q_len=DECODE_MAX_Q_LEN,
                         q_starts=q_starts[: short_requests + 1], context_lens=context_lens[:short_requests],
                         out=out[:short_rows], **common)
@@ -485,7 +489,7 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), width if packed_out else out.stride(0),
                                         _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads,
                                         head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), int(packed_out),
-                                        n_parts, _ptr(parts), _ptr(arrivals), softcap, _ptr(sinks), chunk, _stream()))
+                                        n_parts, _ptr(parts), _ptr(arrivals), softcap, _ptr(sinks), chunk, int(wide_out), _stream()))
         return result
     if (max_q_len is not None and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None
             and rows_aligned and lib.mllm_attention_prefill_supported(head_size, page_size)):
@@ -494,9 +498,9 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         n_requests = context_lens.shape[0]
         _require(q_starts.shape[0] == n_requests + 1, "q_starts must have one entry more than context_lens")
         _require(block_tables.shape[0] >= n_requests, "fewer block tables than requests")
-        check(lib.mllm_attention_prefill(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_starts), _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n_requests, int(max_q_len), int(max_len or 0), n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), chunk, _stream()))
+        check(lib.mllm_attention_prefill(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_starts), _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n_requests, int(max_q_len), int(max_len or 0), n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), chunk, int(wide_out), _stream()))
         return out
-    check(lib.mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), chunk, _stream()))
+    check(lib.mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), softcap, _ptr(sinks), chunk, int(wide_out), _stream()))
     return out
 
 
@@ -1206,21 +1210,24 @@ def map_rows(rows, q_at: int, k_at: int | None, v_at: int | None, q_gain, k_gain
     return out
 
 
-def map_difference(maps_out, gate, lam: float, eps: float, n_heads, n_kv_heads, vdim, head_size, scale: float = 1.0, out=None):
+def map_difference(maps_out, gate, lam: float, eps: float, n_heads, n_kv_heads, vdim, head_size, scale: float = 1.0, out=None, out_dtype=None):
     """Two maps a head into one: with a1, a2 the results of a head's maps in ``maps_out`` ([rows, n_heads * 2 * head_size] as the paged
     attention leaves them for the queries of ``map_rows``; the first ``vdim`` elements of a head count), x = a1 - lam * a2 and out = x /
     sqrt(mean(x^2) + eps) * scale * sigmoid(gate), [rows, n_heads * vdim] of the maps' type, the heads in their own order. ``gate``:
-    float32 rows [rows, n_heads * vdim] (strided; None: no gate)."""
+    float32 rows [rows, n_heads * vdim] (strided; None: no gate). ``out_dtype``: the maps may be float32 (the attention's ``wide_out``)
+    and the result of a narrower type, the one the output product reads; None: the maps' type."""
     _require(maps_out.is_cuda and maps_out.dim() == 2 and maps_out.stride(1) == 1 and maps_out.shape[1] == 2 * n_heads * head_size,
              "the maps' rows do not match the heads")
     n = maps_out.shape[0]
     if gate is not None:
         _rows_f32(gate, "gate", n_heads * vdim)
         _require(gate.shape[0] == n, "the gate's rows do not match")
+    out_dtype = out_dtype or (maps_out.dtype if out is None else out.dtype)
+    _require(maps_out.dtype in (torch.float32, out_dtype), "the maps are float32 or of the result's type")
     if out is None:
-        out = torch.empty((n, n_heads * vdim), dtype=maps_out.dtype, device=maps_out.device)
-    _device_tensor(out, "out", maps_out.dtype, 2)
+        out = torch.empty((n, n_heads * vdim), dtype=out_dtype, device=maps_out.device)
+    _device_tensor(out, "out", out_dtype, 2)
     _require(tuple(out.shape) == (n, n_heads * vdim) and out.stride(1) == 1, "out has the wrong shape")
     check(library().mllm_map_difference(_ptr(maps_out), maps_out.stride(0), _ptr(gate), 0 if gate is None else gate.stride(0), _ptr(out), out.stride(0),
-                                        float(lam), float(eps), float(scale), n, n_heads, n_kv_heads, vdim, head_size, _code(maps_out.dtype), _stream()))
+                                        float(lam), float(eps), float(scale), n, n_heads, n_kv_heads, vdim, head_size, _code(maps_out.dtype), _code(out_dtype), _stream()))
     return out

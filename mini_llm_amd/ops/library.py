@@ -29,10 +29,10 @@ _SIGNATURES = {
     "mllm_probe_read": [P, c_longlong, P, c_int, P],
     "mllm_probe_mfma": [P, c_int, c_int, c_int, P],
     "mllm_cache_write": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
-    "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_float, P, c_int, P],
-    "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, P, P, c_float, P, c_int, P],
+    "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_float, P, c_int, c_int, P],
+    "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, P, P, c_float, P, c_int, c_int, P],
     "mllm_attention_decode_supported": [c_int, c_int, c_int],
-    "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_float, P, c_int, P],
+    "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_float, P, c_int, c_int, P],
     "mllm_attention_prefill_supported": [c_int, c_int],
     "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P, P, P],
     "mllm_gemm_best_per_row": [c_int, c_int, c_int, c_int],
@@ -53,7 +53,7 @@ _SIGNATURES = {
     "mllm_silu_mul": [P, P, c_int, c_int, c_int, P],
     "mllm_map_rows": [P, c_int, c_int, c_int, c_int, P, P, c_float, P, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                       c_int, P],
-    "mllm_map_difference": [P, c_int, P, c_int, P, c_int, c_float, c_float, c_float, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_map_difference": [P, c_int, P, c_int, P, c_int, c_float, c_float, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_heads_linear": [P, c_int, c_int, c_int, P, c_int, P, c_int, c_int, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_latent_attention_supported": [c_int, c_int, c_int],
     "mllm_latent_attention_head_group": [c_int],

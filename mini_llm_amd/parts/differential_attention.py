@@ -16,8 +16,9 @@ it), with queries, mask and everything else of its own.
 
 One product makes everything that reads h ([q | k | v | g], 32-bit sums); ``kernels.map_rows`` norms, rotates and writes the pages;
 the framework's paged attention kernels run the 2 H maps as heads of their own over 2 G key heads (a value head is stored under
-each of its two maps, so that the kernels' grouping of heads serves unchanged); ``kernels.map_difference`` subtracts, norms and
-gates. Heads of different key and value sizes are kept in pages of the larger size (rounded to 16) with zeros behind."""
+each of its two maps, so that the kernels' grouping of heads serves unchanged) and leave their results in 32-bit, because a
+difference of two maps that see nearly the same keys multiplies whatever rounding they carry; ``kernels.map_difference`` subtracts,
+norms and gates. Heads of different key and value sizes are kept in pages of the larger size (rounded to 16) with zeros behind."""
 
 from __future__ import annotations
 
@@ -112,11 +113,11 @@ class DifferentialAttention(Mixer):
             q, ctx.k_pages, ctx.v_pages, batch.token_request, batch.positions, ctx.group.block_tables,
             self.n_heads * MAPS, self.n_kv_heads * MAPS, self.head_size, self.scale, chunk=self.chunk or 0,
             max_q_len=batch.max_q_len, max_len=batch.max_total_len, q_starts=batch.q_starts, context_lens=batch.context_lens,
-            first_row=getattr(batch, "first_row", 0),
+            first_row=getattr(batch, "first_row", 0), wide_out=True,
             **({"short_rows": batch.short_rows, "short_requests": batch.short_requests} if batch.short_portion <= kernels.DECODE_MAX_Q_LEN else {}),
         )
         mixed = kernels.map_difference(maps_out, fused[:, g_at : g_at + self.g_width], self.lam, self.eps, self.n_heads, self.n_kv_heads, self.vdim,
-                                       self.head_size, scale=1.0 - self.diff)
+                                       self.head_size, scale=1.0 - self.diff, out_dtype=x.dtype)
         return self._out_product(mixed, self.o, residual)
 
 

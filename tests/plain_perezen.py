@@ -227,3 +227,55 @@ def tensor_shapes(config: dict) -> dict:
             shapes[p + "norm2"] = shapes[p + "norm2b"] = (width,)
             shapes.update({p + "mlp.gate": (ff, width), p + "mlp.up": (ff, width), p + "mlp.down": (width, ff)})
     return shapes
+
+
+def greedy(config: dict, tensors: dict, prompt, n_new: int, round_to=None) -> list:
+    tokens = list(prompt)
+    for _ in range(n_new):
+        tokens.append(int(forward(config, tensors, tokens, round_to)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+# -- random models for the tests ------------------------------------------------------------------------------------------
+def random_weights(config: dict, seed: int) -> dict:
+    """Weights whose activations stay of order one: matrices ~ N(0, 1/in), gains around one, biases of order one, forget biases well
+    above zero, the four vectors of the second map's weight small. float32 arrays holding bfloat16 values (as files hold them)."""
+    import plain_gpt2
+
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shape in tensor_shapes(config).items():
+        last = name.rsplit(".", 1)[-1]
+        if name.endswith(".f.b"):
+            value = rng.normal(3.0, 0.5, shape)
+        elif last in ("lq1", "lk1", "lq2", "lk2"):
+            value = rng.normal(0.0, 0.25, shape)
+        elif last in ("norm", "norm1", "norm2", "norm1b", "norm2b"):
+            value = 1.0 + rng.normal(0.0, 0.1, shape)
+        elif last == "b":
+            value = rng.normal(0.0, 0.3, shape)
+        elif name == "embed":
+            value = rng.normal(0.0, 1.0, shape)
+        elif name == "pos":
+            value = rng.normal(0.0, 0.3, shape)
+        else:
+            value = rng.normal(0.0, shape[1] ** -0.5, shape)
+        out[name] = plain_gpt2.round_to_bf16(np.asarray(value, dtype=np.float32))
+    return out
+
+
+def as_float64(weights: dict) -> dict:
+    return {name: np.asarray(value, dtype=np.float64) for name, value in weights.items()}
+
+
+def write_model_dir(path, config: dict, weights: dict):
+    import json
+    from pathlib import Path
+
+    import plain_gpt2
+
+    path = Path(path)
+    path.mkdir(parents=True, exist_ok=True)
+    (path / "config.json").write_text(json.dumps(config, indent=1))
+    plain_gpt2.write_safetensors(path / "model.safetensors", {k: np.asarray(v, dtype=np.float32) for k, v in weights.items()}, bf16=True)
+    return path
