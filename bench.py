@@ -340,7 +340,7 @@ _KERNEL_CLASSES = {
     "products": ("gemm", "gemm_split", "gemm_qkv_cache", "gemm_best", "heads_linear"),
     "attention": ("attention", "attention_decode", "attention_prefill", "latent_attention"),
     "row-wise": ("layernorm", "pending_layernorm", "rms_norm", "head_norm", "latent_rows", "silu_mul", "pending_sum", "add", "cache_write", "embed",
-                 "projection_rows", "head_gate", "gated_norm", "short_conv"),
+                 "projection_rows", "head_gate", "gated_norm", "short_conv", "map_rows", "map_difference"),
     "recurrence": ("recurrence",),
     "layer kernels": ("decode_attention_half", "decode_mlp_half"),
     "choice": ("choose", "sample"),
@@ -391,9 +391,28 @@ def ketolix_shape(width: int, layers: int, vocab: int = 50257) -> dict:
     return {"architecture": "Ketolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": [pattern[i % 4] for i in range(layers)]}
 
 
+def perezen_shape(width: int, layers: int, vocab: int = 50257) -> dict:
+    """Layers in fours: a matrix memory (heads of 64 x 128, as Ketolix's), then three layers of differential attention (width / 128 heads
+    of two maps of 64 and values of 128, a key/value head for every two, chunks of 512 positions, all of a map rotated), of which the
+    second reads the keys and values the first keeps; feed-forwards of 8/3 x width; a position table of the context's length."""
+    heads, wide_heads = max(1, width // 128), max(1, width // 128)
+    ff = -(-(8 * width // 3) // 64) * 64
+    mlp = {"kind": "dense", "ff": ff}
+    mixer = {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 64, "vdim": 128, "scale": 0.125, "diff": 0.5, "mask": {"size": 512},
+             "rot": {"dims": 64, "base": 10000.0}}
+    memory = {"type": "mlstm", "mlp": mlp, "mixer": {"heads": wide_heads, "dim": 64, "vdim": 128, "gate_cap": 15.0}}
+    out = []
+    for index in range(layers):
+        if index % 4 == 0:
+            out.append(memory)
+        else:
+            out.append({"type": "attention", "mlp": mlp, "mixer": dict(mixer, kv_from=index - 1) if index % 4 == 2 else mixer})
+    return {"architecture": "Perezen", "vocab": vocab, "width": width, "max_positions": CONTEXT, "norm": {"eps": 1e-5}, "logit_scale": 1.0, "layers": out}
+
+
 def measure_design(args) -> dict:
     """Prefill and decode throughput of a design and of the framework's closest older model with as many layers of the same width
-    (random weights): Gimozen beside GPT-2, Ketolix beside Gimozen; and where each model's step spends its time, by class of
+    (random weights): Gimozen beside GPT-2, Ketolix beside Gimozen, Perezen beside Ketolix; and where each model's step spends its time, by class of
     kernel, inside a prompt step and a decode step."""
     import numpy as np
     import torch
@@ -403,7 +422,9 @@ def measure_design(args) -> dict:
     from mini_llm_amd.engine.engine import Engine, EngineOptions
 
     width, layers = DESIGN_SIZES[args.shape]
-    if args.design == "ketolix":
+    if args.design == "perezen":
+        raws = {"perezen": perezen_shape(width, layers), "ketolix": ketolix_shape(width, layers)}
+    elif args.design == "ketolix":
         raws = {"ketolix": ketolix_shape(width, layers), "gimozen": gimozen_shape(width, layers)}
     else:
         raws = {"gimozen": gimozen_shape(width, layers),
@@ -668,8 +689,8 @@ def main() -> int:
     parser.add_argument("--serving", action="store_true", help="continuous batching of 64 requests on the GPT-2 medium shape through the scheduler")
     parser.add_argument("--temperature", type=float, default=0.0, help="sampling temperature of --serving (0: greedy)")
     parser.add_argument("--step-by-step", action="store_true", help="--serving reads every step's tokens before it launches the next")
-    parser.add_argument("--design", default=None, choices=("gimozen", "ketolix"), help="a design beside the closest older model with as many layers of the same width "
-                        "(--shape small|medium): Gimozen beside GPT-2, Ketolix beside Gimozen; prefill and decode throughput of both, and where their steps spend the time")
+    parser.add_argument("--design", default=None, choices=("gimozen", "ketolix", "perezen"), help="a design beside the closest older model with as many layers of the same width "
+                        "(--shape small|medium): Gimozen beside GPT-2, Ketolix beside Gimozen, Perezen beside Ketolix; prefill and decode throughput of both, and where their steps spend the time")
     parser.add_argument("--peaks", action="store_true", help="measure this machine's read bandwidth and matrix-core rate with the library's probes")
     args = parser.parse_args()
     if args.gpus != 1:

@@ -21,13 +21,15 @@ __device__ __forceinline__ void store_from_float(void* base, size_t index, int c
 // given, names the input row of each output row. The result goes to `stream` (32-bit, what the residual stream goes on
 // with) and / or `rows` (the element type the next product reads); either may be null. `residual` (32-bit, the output's
 // shape), if given, is added to the normed rows: out = residual + norm(h) g, the sum of a layer whose norm sits on its
-// branch's output.
+// branch's output. `next_weight`, if given (rows of up to 64 * REGS elements): `rows` are not the result itself but the result normed
+// once more, out / sqrt(mean(out^2) + eps) * next_weight (or 1 + next_weight): what the norm in front of the next branch would
+// make of the new stream, so that a layer with a norm behind one branch and another in front of the next runs one kernel for both.
 template <int REGS>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const void* __restrict__ y, int y_code, float alpha,
                                                        const int* __restrict__ row_index, const float* __restrict__ weight, int one_plus,
                                                        float eps, float* __restrict__ stream, void* __restrict__ rows, int rows_code,
                                                        int n_rows, int width, int n_partials, long long partial_stride,
-                                                       const float* __restrict__ residual) {
+                                                       const float* __restrict__ residual, const float* __restrict__ next_weight) {
     const int lane = threadIdx.x % WAVE;
     const int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
     if (row >= n_rows) return;
@@ -36,13 +38,14 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
     const float plus = one_plus ? 1.0f : 0.0f;
     if constexpr (REGS > 0) {
         // everything is asked for at once, from clamped places, so that the wave waits for memory once
-        float kept[REGS], added[REGS], gains[REGS], base[REGS];
+        float kept[REGS], added[REGS], gains[REGS], base[REGS], next_gains[REGS];
 #pragma unroll
         for (int r = 0; r < REGS; r++) {
             const int i = min(lane + r * WAVE, width - 1);
             kept[r] = x[in_at + i];
             gains[r] = weight[i];
             base[r] = residual ? residual[out_at + i] : 0.0f;
+            next_gains[r] = next_weight ? next_weight[i] : 0.0f;
         }
         if (y) {
             if (y_code == MLLM_F32) {
@@ -78,6 +81,25 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
             squares += h * h;
         }
         const float inverse = 1.0f / sqrtf(wave_total(squares) / (float)width + eps);
+        if (next_weight) {   // (the same for all waves of the launch)
+            float again = 0.0f;
+#pragma unroll
+            for (int r = 0; r < REGS; r++) {
+                const float value = lane + r * WAVE < width ? base[r] + kept[r] * inverse * (plus + gains[r]) : 0.0f;
+                kept[r] = value;
+                again += value * value;
+            }
+            const float next_inverse = 1.0f / sqrtf(wave_total(again) / (float)width + eps);
+#pragma unroll
+            for (int r = 0; r < REGS; r++) {
+                const int i = lane + r * WAVE;
+                if (i < width) {
+                    if (stream) stream[out_at + i] = kept[r];
+                    if (rows) store_from_float(rows, out_at + i, rows_code, kept[r] * next_inverse * (plus + next_gains[r]));
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < REGS; r++) {
             const int i = lane + r * WAVE;
@@ -311,7 +333,7 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ bot
 
 MLLM_API int mllm_rms_norm(const float* x, const void* y, int y_dtype, float alpha, const int* row_index, const float* weight, int one_plus,
                            float eps, float* stream_out, void* rows_out, int rows_dtype, int n_rows, int width, int n_partials,
-                           long long partial_stride, const float* residual, hipStream_t stream) {
+                           long long partial_stride, const float* residual, const float* next_weight, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && width > 0, "rms_norm: bad sizes rows=%d width=%d", n_rows, width);
     MLLM_REQUIRE(x != nullptr && weight != nullptr && (stream_out != nullptr || rows_out != nullptr), "rms_norm: a missing operand");
     MLLM_REQUIRE(y == nullptr || y_dtype == MLLM_F32 || y_dtype == MLLM_BF16, "rms_norm: unknown element type of the addend");
@@ -319,10 +341,11 @@ MLLM_API int mllm_rms_norm(const float* x, const void* y, int y_dtype, float alp
     MLLM_REQUIRE(y == nullptr || row_index == nullptr, "rms_norm: gathered rows take no addend");
     MLLM_REQUIRE(n_partials >= 1 && (n_partials == 1 || (y != nullptr && y_dtype == MLLM_F32 && partial_stride >= (long long)n_rows * width)),
                  "rms_norm: partial products are 32-bit and lie a whole matrix apart");
+    MLLM_REQUIRE(next_weight == nullptr || (width <= 2048 && rows_out != nullptr), "rms_norm: a second norm takes rows of up to 2048 elements and writes `rows`");
     if (n_rows == 0) return 0;
     const int waves = 4, blocks = ceil_div(n_rows, waves);
     mllm_count_kernel(MLLM_K_RMS_NORM);
-#define LAUNCH(REGS) rms_norm_kernel<REGS><<<blocks, 64 * waves, 0, stream>>>(x, y, y_dtype, alpha, row_index, weight, one_plus, eps, stream_out, rows_out, rows_dtype, n_rows, width, n_partials, partial_stride, residual)
+#define LAUNCH(REGS) rms_norm_kernel<REGS><<<blocks, 64 * waves, 0, stream>>>(x, y, y_dtype, alpha, row_index, weight, one_plus, eps, stream_out, rows_out, rows_dtype, n_rows, width, n_partials, partial_stride, residual, next_weight)
     if (width <= 256) LAUNCH(4);
     else if (width <= 512) LAUNCH(8);
     else if (width <= 1024) LAUNCH(16);

@@ -40,6 +40,8 @@ def build_perezen(config: PerezenConfig, precision) -> Model:
         ))
         borrowed = getattr(layer.mixer, "kv_from", None)
         schedule.append(LayerCall(block=index, cache=index if borrowed is None else borrowed, write_cache=borrowed is None))
+    for block, following in zip(blocks, blocks[1:]):   # the schedule runs the layers in their order: a layer's last kernel norms for the next
+        block.hand_to(following.norm_1)
     return Model(
         config, precision,
         embedding=TokenEmbedding(config.vocab, width, tensor_name="", std=1.0),

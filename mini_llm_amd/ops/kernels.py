@@ -727,9 +727,24 @@ class NormedRows:
         return self.stream.shape
 
 
+@dataclass
+class ReadyRows:
+    """Rows of the residual stream in float32 (``stream``) and, made ahead of time by the kernel that wrote them, the rows that the
+    norm ``norm`` (a part) makes of them, in the element type the next products read (``rows``). A layer whose last norm sits on a
+    branch's output hands these to the layer whose first norm is ``norm``; any other reader takes ``stream``."""
+
+    stream: torch.Tensor
+    rows: torch.Tensor
+    norm: object
+
+    @property
+    def shape(self):
+        return self.stream.shape
+
+
 def settle(hidden):
     """The stream as plain float32 rows: a tensor as it is, pending rows with their sums taken."""
-    if isinstance(hidden, NormedRows):
+    if isinstance(hidden, (NormedRows, ReadyRows)):
         return hidden.stream
     if not isinstance(hidden, PendingRows):
         return hidden
@@ -826,14 +841,20 @@ def decode_mlp_half(hidden, gamma, beta, eps, w_up, b_up, w_down, b_down, activa
 
 
 # -- layers that norm after the sum, norm their heads, gate their feed-forward, or keep a latent -----------------
+RMS_NORM_TWICE_WIDTH = 2048   # the widest rows that one launch norms twice (they stay in a wave's registers between the two)
+
+
 def rms_norm(x, weight, eps, *, addend=None, alpha: float = 1.0, one_plus: bool = False, out_dtype=None, row_index=None, with_stream: bool = False,
-             residual=None):
+             residual=None, next_weight=None):
     """h / sqrt(mean(h^2) + eps) * g over rows of h = alpha * x (+ addend), g = weight or, with ``one_plus``, 1 + weight.
     x: float32 [rows, width]; addend: float32 or bfloat16 of the same shape, or float32 [n, rows, width], the partial products
     of a product cut along K (``linear_split``), whose sum is the addend; weight: float32 [width]. ``row_index`` (int32)
     picks the input row of each output row. ``residual`` (float32, the output's shape) is added to the normed rows: residual +
     norm(h) * g, the sum of a layer whose norm sits on its branch's output. Returns the rows in ``out_dtype``, or with ``with_stream`` (the rows in float32:
-    what a residual stream goes on with, the rows in ``out_dtype``); ``out_dtype`` None: the float32 rows alone."""
+    what a residual stream goes on with, the rows in ``out_dtype``); ``out_dtype`` None: the float32 rows alone.
+    ``next_weight`` (float32 [width]; with ``with_stream`` and an ``out_dtype``, rows of up to RMS_NORM_TWICE_WIDTH elements): the rows in
+    ``out_dtype`` are the result normed once more with this gain vector, r / sqrt(mean(r^2) + eps) * g', while the float32 rows are the
+    result r itself: the norm behind one branch and the norm in front of the next from one kernel."""
     _device_tensor(x, "x", torch.float32, 2)
     _device_tensor(weight, "weight", torch.float32, 1)
     width = x.shape[1]
@@ -853,11 +874,15 @@ def rms_norm(x, weight, eps, *, addend=None, alpha: float = 1.0, one_plus: bool 
     if residual is not None:
         _device_tensor(residual, "residual", torch.float32, 2)
         _require(tuple(residual.shape) == (n, width), "the residual must have the output's shape")
+    if next_weight is not None:
+        _device_tensor(next_weight, "next_weight", torch.float32, 1)
+        _require(next_weight.shape[0] == width and width <= RMS_NORM_TWICE_WIDTH and with_stream and out_dtype is not None,
+                 "a second norm takes rows of up to 2048 elements, its own gain vector, and leaves both the stream and the normed rows")
     stream = torch.empty((n, width), dtype=torch.float32, device=x.device) if with_stream or out_dtype is None else None
     rows = torch.empty((n, width), dtype=out_dtype, device=x.device) if out_dtype is not None else None
     check(library().mllm_rms_norm(_ptr(x), _ptr(addend), 0 if addend is None else _code(addend.dtype), float(alpha), _ptr(row_index), _ptr(weight),
                                   int(bool(one_plus)), float(eps), _ptr(stream), _ptr(rows), 0 if rows is None else _code(rows.dtype), n, width, n_partials,
-                                  partial_stride, _ptr(residual), _stream()))
+                                  partial_stride, _ptr(residual), _ptr(next_weight), _stream()))
     if out_dtype is None:
         return stream
     return (stream, rows) if with_stream else rows

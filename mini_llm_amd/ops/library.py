@@ -47,7 +47,7 @@ _SIGNATURES = {
     "mllm_linear_split_static": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_static_scratch_prepare": [],
     "mllm_pending_layernorm": [P, P, P, c_int, c_int, P, P, P, P, P, c_int, c_int, c_float, c_int, c_int, P],
-    "mllm_rms_norm": [P, P, c_int, c_float, P, P, c_int, c_float, P, P, c_int, c_int, c_int, c_int, c_longlong, P, P],
+    "mllm_rms_norm": [P, P, c_int, c_float, P, P, c_int, c_float, P, P, c_int, c_int, c_int, c_int, c_longlong, P, P, P],
     "mllm_head_norm": [P, c_int, P, P, c_float, c_float, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_latent_rows": [P, c_int, P, c_int, P, c_float, P, c_float, c_int, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_silu_mul": [P, P, c_int, c_int, c_int, P],

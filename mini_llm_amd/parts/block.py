@@ -100,7 +100,12 @@ class SandwichNormBlock(Block):
     """A norm in front of each branch and one on its output: x <- x + norm_1b(mixer(norm_1(x))), then x <- x + norm_2b(feed_forward(norm_2(x))).
     ``feed_forward`` None: the layer ends behind its mixer. The stream is float32 rows; the norms on the outputs have ``forward_added``
     (RMSNorm: stream + norm(branch) from one kernel, which also adds up the partial products of a branch whose last product was cut
-    along K), and mixer and feed-forward return their branch alone when given no residual."""
+    along K, and norms the sum once more for the branch that follows), and mixer and feed-forward return their branch alone when given
+    no residual. ``hand_to(norm)``: the norm that reads this layer's output next (the following layer's ``norm_1``); the layer then
+    returns kernels.ReadyRows, its stream and what that norm makes of it, and a layer that is handed such rows made by its own
+    ``norm_1`` does not run it again. A layer is so two norm kernels for a branch's four norms."""
+
+    takes_pending = True   # takes plain rows, pending rows or the ReadyRows of the layer before
 
     def __init__(self, norm_1: Norm, mixer: Mixer, norm_1b: Norm, norm_2: Norm | None, feed_forward: FeedForward | None, norm_2b: Norm | None,
                  compute_dtype, names=("norm1", "mix.", "norm1b", "norm2", "mlp.", "norm2b")):
@@ -109,6 +114,7 @@ class SandwichNormBlock(Block):
         self.norm_1, self.mixer, self.norm_1b, self.norm_2, self.feed_forward, self.norm_2b = norm_1, mixer, norm_1b, norm_2, feed_forward, norm_2b
         self.compute_dtype = compute_dtype
         self._names = names
+        self._following = None
 
     def children(self):
         parts = dict(zip(self._names, (self.norm_1, self.mixer, self.norm_1b, self.norm_2, self.feed_forward, self.norm_2b)))
@@ -117,13 +123,26 @@ class SandwichNormBlock(Block):
     def mixer_part(self):
         return self.mixer
 
+    def hand_to(self, norm: Norm | None):
+        self._following = norm
+
+    def _added(self, norm, stream, branch, then):
+        if then is None or not hasattr(norm, "forward_added"):
+            return norm.forward_added(stream, branch)
+        return norm.forward_added(stream, branch, then=then, out_dtype=self.compute_dtype)
+
     def forward(self, hidden, ctx: LayerContext):
-        branch = self.mixer.forward(self.norm_1.forward(hidden, self.compute_dtype), None, ctx)
-        hidden = self.norm_1b.forward_added(hidden, branch)
+        from ..ops import kernels
+
+        if isinstance(hidden, kernels.ReadyRows) and hidden.norm is self.norm_1:
+            stream, rows = hidden.stream, hidden.rows
+        else:
+            stream = kernels.settle(hidden)
+            rows = self.norm_1.forward(stream, self.compute_dtype)
+        hidden = self._added(self.norm_1b, stream, self.mixer.forward(rows, None, ctx), self.norm_2 if self.feed_forward is not None else self._following)
         if self.feed_forward is None:
             return hidden
-        branch = self.feed_forward.forward(self.norm_2.forward(hidden, self.compute_dtype), None)
-        return self.norm_2b.forward_added(hidden, branch)
+        return self._added(self.norm_2b, hidden.stream, self.feed_forward.forward(hidden.rows, None), self._following)
 
 
 register_part("block", "pre_norm", PreNormBlock)

@@ -67,13 +67,23 @@ class RMSNorm(Norm):
         return kernels.NormedRows(*kernels.rms_norm(x, self.weight, self.eps, addend=addend, alpha=alpha, one_plus=self.one_plus,
                                                     out_dtype=out_dtype, with_stream=True))
 
-    def forward_added(self, stream, branch):
+    def forward_added(self, stream, branch, then=None, out_dtype=None):
         """stream + norm(branch) in float32 alone: for a layer whose next branch has a norm of its own in front. ``branch`` as for
-        ``forward_onto``."""
+        ``forward_onto``. ``then``: that next norm (an RMSNorm with the same eps and kind of gain, rows the kernel norms twice in one
+        launch) and the element type its products read: the result is kernels.ReadyRows(sum, then(sum), then), from the one kernel."""
         addend = None
         if branch.dim() == 3:
             branch, addend = branch[0], (branch[1:] if branch.shape[0] > 1 else None)
-        return kernels.rms_norm(branch, self.weight, self.eps, addend=addend, one_plus=self.one_plus, residual=stream)
+        if then is None:
+            return kernels.rms_norm(branch, self.weight, self.eps, addend=addend, one_plus=self.one_plus, residual=stream)
+        if (isinstance(then, RMSNorm) and then.eps == self.eps and then.one_plus == self.one_plus and then.width == self.width
+                and self.width <= kernels.RMS_NORM_TWICE_WIDTH):
+            total, rows = kernels.rms_norm(branch, self.weight, self.eps, addend=addend, one_plus=self.one_plus, residual=stream, out_dtype=out_dtype,
+                                           with_stream=True, next_weight=then.weight)
+        else:
+            total = kernels.rms_norm(branch, self.weight, self.eps, addend=addend, one_plus=self.one_plus, residual=stream)
+            rows = then.forward(total, out_dtype)
+        return kernels.ReadyRows(total, rows, then)
 
     def forward_onto(self, stream, branch, out_dtype):
         """stream + norm(branch) -> kernels.NormedRows: the sum of a layer whose norm sits on its branch's output, in float32 and in

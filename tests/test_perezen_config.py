@@ -40,6 +40,8 @@ def test_round_trip_tensor_names_cache_and_state(name):
         else:
             assert index not in state
     assert built.all_graph_safe() and built.max_positions() == raw["max_positions"]
+    # every layer but the last knows the norm that reads its output next
+    assert all(a._following is b.norm_1 for a, b in zip(built.blocks, built.blocks[1:])) and built.blocks[-1]._following is None
 
 
 def test_what_the_configuration_refuses():

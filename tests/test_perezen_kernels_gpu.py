@@ -245,3 +245,28 @@ def test_learned_positions_join_the_token_rows_unscaled():
         got = k.embed(ints(tokens), ints(positions), gpu(table, dtype), gpu(pos, dtype))
         np.testing.assert_allclose(got.float().cpu().numpy(), rounded(table, dtype)[tokens] + rounded(pos, dtype)[positions], atol=1e-6)
         assert got.dtype == torch.float32    # the stream is 32-bit whatever the tables are
+
+
+@pytest.mark.parametrize("width", [5, 64, 100, 768, 2048, 2500])
+def test_the_norm_behind_a_branch_and_the_norm_in_front_of_the_next_from_one_kernel(width):
+    from mini_llm_amd.parts import make_part
+
+    rng = np.random.default_rng(width)
+    stream, branch = rng.normal(0, 2, (7, width)), rng.normal(0, 3, (7, width))
+    w, w_next = rng.normal(1, 0.3, width), rng.normal(1, 0.3, width)
+    total = stream + plain.rms_unit(branch, 1e-5) * w
+    behind, ahead = (make_part("norm", "rmsnorm", width=width, eps=1e-5, tensor_name="") for _ in range(2))
+    behind.bind({"": gpu(w)})
+    ahead.bind({"": gpu(w_next)})
+    for dtype in DTYPES:
+        got = behind.forward_added(gpu(stream), gpu(branch), then=ahead, out_dtype=dtype)    # (rows of 2,500 take two launches)
+        assert got.norm is ahead and got.rows.dtype == dtype
+        np.testing.assert_allclose(got.stream.cpu().numpy(), total, atol=2e-5, rtol=2e-5)
+        np.testing.assert_allclose(got.rows.float().cpu().numpy(), plain.rms_unit(total, 1e-5) * w_next, **tol(dtype))
+    # the branch as the partial products of a product cut along K
+    parts = rng.normal(0, 1, (4, 7, width))
+    got = behind.forward_added(gpu(stream), gpu(parts), then=ahead, out_dtype=torch.float32)
+    total = stream + plain.rms_unit(parts.sum(axis=0), 1e-5) * w
+    np.testing.assert_allclose(got.stream.cpu().numpy(), total, atol=2e-5, rtol=2e-5)
+    np.testing.assert_allclose(got.rows.cpu().numpy(), plain.rms_unit(total, 1e-5) * w_next, atol=3e-5, rtol=3e-5)
+    np.testing.assert_allclose(behind.forward_added(gpu(stream), gpu(parts)).cpu().numpy(), total, atol=2e-5, rtol=2e-5)
