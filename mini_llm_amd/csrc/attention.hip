@@ -676,7 +676,9 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
         }
         // ---- scale, mask (only where the tile touches the diagonal, a window or the tile's end), maximum ----
         float tile_max = -INFINITY;
-        const bool interior = wave_full && !masked_from && k0 + PF_KEYS - 1 <= wave_first_position;
+        // all queries of the wave see all keys of the tile: it lies before the first query and not before the last query's first key
+        const bool interior = wave_full && k0 + PF_KEYS - 1 <= wave_first_position &&
+                              (!masked_from || k0 >= first_visible_key(wave_last_position, window, options.chunk));
         if (interior) {
 #pragma unroll
             for (int j = 0; j < 2; j++)
