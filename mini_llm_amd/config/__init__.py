@@ -1,4 +1,5 @@
 from .base import ConfigError, ModelConfig, read_config_json
+from .dizizen import DizizenConfig
 from .gimozen import GimozenConfig
 from .gpt2 import GPT2Config
 from .ketolix import KetolixConfig
@@ -16,6 +17,7 @@ from .registry import (
 __all__ = [
     "Architecture",
     "ConfigError",
+    "DizizenConfig",
     "GimozenConfig",
     "GPT2Config",
     "KetolixConfig",

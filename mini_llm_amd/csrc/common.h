@@ -69,7 +69,7 @@ enum MllmKernel : int {
     MLLM_K_STATIC_SUM, MLLM_K_PROBE, MLLM_K_SAMPLE, MLLM_K_GEMM_BEST, MLLM_K_CHOOSE, MLLM_K_RMS_NORM, MLLM_K_HEAD_NORM,
     MLLM_K_LATENT_ROWS, MLLM_K_SILU_MUL, MLLM_K_HEADS_LINEAR, MLLM_K_LATENT_ATTENTION, MLLM_K_LATENT_MERGE, MLLM_K_PROJECTION_ROWS,
     MLLM_K_HEAD_GATE, MLLM_K_GATED_NORM, MLLM_K_SHORT_CONV, MLLM_K_RECURRENCE, MLLM_K_MAP_ROWS,
-    MLLM_K_MAP_DIFFERENCE, MLLM_K_KINDS
+    MLLM_K_MAP_DIFFERENCE, MLLM_K_TURN_HEADS, MLLM_K_GATE_UNIT, MLLM_K_ROUTE, MLLM_K_EXPERT_UNIT, MLLM_K_BRANCH_JOIN, MLLM_K_KINDS
 };
 void mllm_count_kernel(MllmKernel kind);
 

@@ -23,6 +23,37 @@ __device__ __forceinline__ void turned(float u, float v, int position, double fr
     b = v * c + u * s;
 }
 
+// Element d (< rot_dims) of a head `in` after its pair has turned by sign x position x frequencies[pair]: pairs are (m, m + rot_dims / 2)
+// or, with `neighbours`, (2m, 2m + 1).
+__device__ __forceinline__ float turned_element(const float* in, int d, int rot_dims, int neighbours, int position, const double* frequencies, float sign) {
+    const int half = rot_dims / 2;
+    const bool first = neighbours ? (d & 1) == 0 : d < half;
+    const int pair = neighbours ? d / 2 : (first ? d : d - half);
+    const int other = neighbours ? d ^ 1 : (first ? d + half : d - half);
+    float a, b;
+    if (first) turned(in[d], in[other], position, sign * frequencies[pair], a, b);
+    else turned(in[other], in[d], position, sign * frequencies[pair], b, a);
+    return a;
+}
+
+// A wave per (row, head): the first rot_dims elements of the head turned by sign x position x frequencies[pair] (sign -1 turns back what
+// turned_element with sign 1 turned), the elements behind them up to out_size copied. `in` heads lie in_size apart (float32 rows), `out`
+// heads out_size apart, so that heads kept wider than their values leave at the values' own size.
+template <typename T>
+__global__ __launch_bounds__(64 * MAP_WAVES) void turn_heads_kernel(const float* __restrict__ in, int in_stride, T* __restrict__ out, int out_stride,
+                                                                   const double* __restrict__ frequencies, int rot_dims, int neighbours, float sign,
+                                                                   const int* __restrict__ positions, int n_rows, int n_heads, int in_size, int out_size) {
+    const int lane = threadIdx.x % WAVE;
+    const long long item = (long long)blockIdx.x * MAP_WAVES + threadIdx.x / WAVE;
+    if (item >= (long long)n_rows * n_heads) return;
+    const int row = (int)(item / n_heads), head = (int)(item % n_heads);
+    const float* from = in + (size_t)row * in_stride + (size_t)head * in_size;
+    T* to = out + (size_t)row * out_stride + (size_t)head * out_size;
+    const int position = positions[row];
+    for (int d = lane; d < out_size; d += WAVE)
+        to[d] = from_float<T>(d < rot_dims ? turned_element(from, d, rot_dims, neighbours, position, frequencies, sign) : from[d]);
+}
+
 // A wave per (row, item); a row's items are its n_heads * maps queries, then (where the layer keeps keys and values of its own: k_at
 // >= 0) its n_kv_heads * maps keys and its n_kv_heads values. `rows` are the 32-bit sums of the product that made them, [.. | q | k |
 // v | ..] at columns q_at, k_at, v_at: q as [n_heads, maps, dim], k as [n_kv_heads, maps, dim], v as [n_kv_heads, vdim].
@@ -30,12 +61,14 @@ __device__ __forceinline__ void turned(float u, float v, int position, double fr
 // rot_dims elements i and i + rot_dims / 2 turned as a pair by position x frequencies[i]. Queries go to q_out [row, n_kv_heads, maps, R,
 // head_size], keys to head g * maps + m of the row's slot in k_pages, a value to heads g * maps + 0 .. maps - 1 of v_pages, zeros
 // beyond dim / vdim up to head_size. Padding rows (slot < 0) store nothing.
+// v_frequencies (null: values are kept as they are): of a value's first v_rot_dims elements every pair turns by position x
+// v_frequencies[pair] before it is stored; v_neighbours 0 pairs element m with m + v_rot_dims / 2, 1 pairs 2m with 2m + 1.
 template <typename T>
 __global__ __launch_bounds__(64 * MAP_WAVES) void map_rows_kernel(
     const float* __restrict__ rows, int stride, int q_at, int k_at, int v_at, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
     float eps, const double* __restrict__ frequencies, int rot_dims, const int* __restrict__ positions, const int* __restrict__ slots,
     T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages, int n_rows, int n_heads, int n_kv_heads, int maps, int dim,
-    int vdim, int head_size, int page_size) {
+    int vdim, int head_size, int page_size, const double* __restrict__ v_frequencies, int v_rot_dims, int v_neighbours) {
     const int lane = threadIdx.x % WAVE;
     const int n_q = n_heads * maps, n_k = k_at >= 0 ? n_kv_heads * maps : 0, n_v = k_at >= 0 ? n_kv_heads : 0;
     const int per_row = n_q + n_k + n_v;
@@ -49,9 +82,14 @@ __global__ __launch_bounds__(64 * MAP_WAVES) void map_rows_kernel(
         if (slot < 0) return;
         const int g = which - n_q - n_k;
         const float* in = in_row + v_at + (size_t)g * vdim;
+        const int position = v_frequencies ? positions[row] : 0;
         for (int m = 0; m < maps; m++) {
             T* out = v_pages + (((size_t)(slot / page_size) * (n_kv_heads * maps) + g * maps + m) * page_size + slot % page_size) * head_size;
-            for (int d = lane; d < head_size; d += WAVE) out[d] = from_float<T>(d < vdim ? in[d] : 0.0f);
+            for (int d = lane; d < head_size; d += WAVE) {
+                float value = d < vdim ? in[d] : 0.0f;
+                if (v_frequencies && d < v_rot_dims) value = turned_element(in, d, v_rot_dims, v_neighbours, position, v_frequencies, 1.0f);
+                out[d] = from_float<T>(value);
+            }
         }
         return;
     }
@@ -133,7 +171,7 @@ __global__ __launch_bounds__(64 * MAP_WAVES) void map_difference_kernel(
 MLLM_API int mllm_map_rows(const float* rows, int stride, int q_at, int k_at, int v_at, const float* q_gain, const float* k_gain, float eps,
                            const double* frequencies, int rot_dims, const int* positions, const int* slots, void* q_out, void* k_pages,
                            void* v_pages, int n_rows, int n_heads, int n_kv_heads, int maps, int dim, int vdim, int head_size, int page_size,
-                           int dtype, hipStream_t stream) {
+                           int dtype, const double* v_frequencies, int v_rot_dims, int v_neighbours, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && n_heads > 0 && n_kv_heads > 0 && maps > 0 && dim > 0 && vdim > 0 && page_size > 0, "map_rows: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "map_rows: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(head_size >= dim && head_size >= vdim, "map_rows: heads of %d do not hold %d / %d elements", head_size, dim, vdim);
@@ -143,12 +181,13 @@ MLLM_API int mllm_map_rows(const float* rows, int stride, int q_at, int k_at, in
     MLLM_REQUIRE(k_at < 0 || (v_at >= 0 && k_at + n_kv_heads * maps * dim <= stride && v_at + n_kv_heads * vdim <= stride && slots != nullptr &&
                               k_pages != nullptr && v_pages != nullptr),
                  "map_rows: keys and values to keep need their columns, slots and pages");
+    MLLM_REQUIRE(v_frequencies == nullptr || (v_rot_dims >= 0 && v_rot_dims % 2 == 0 && v_rot_dims <= vdim), "map_rows: %d turned elements of a value of %d", v_rot_dims, vdim);
     if (n_rows == 0) return 0;
     const long long items = (long long)n_rows * (n_heads * maps + (k_at >= 0 ? n_kv_heads * (maps + 1) : 0));
     const int blocks = (int)((items + MAP_WAVES - 1) / MAP_WAVES);
     mllm_count_kernel(MLLM_K_MAP_ROWS);
 #define MAP_ROWS_ARGS(T) rows, stride, q_at, k_at, v_at, q_gain, k_gain, eps, frequencies, rot_dims, positions, slots, (T*)q_out, (T*)k_pages, \
-                         (T*)v_pages, n_rows, n_heads, n_kv_heads, maps, dim, vdim, head_size, page_size
+                         (T*)v_pages, n_rows, n_heads, n_kv_heads, maps, dim, vdim, head_size, page_size, v_frequencies, v_rot_dims, v_neighbours
     if (dtype == MLLM_F32) map_rows_kernel<float><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_ROWS_ARGS(float));
     else if (dtype == MLLM_BF16) map_rows_kernel<bf16_t><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_ROWS_ARGS(bf16_t));
     else MLLM_REQUIRE(false, "map_rows: unknown dtype %d", dtype);
@@ -177,4 +216,22 @@ MLLM_API int mllm_map_difference(const void* maps_out, int maps_stride, const fl
     else MLLM_REQUIRE(false, "map_difference: maps of dtype %d into rows of dtype %d", in_dtype, dtype);
 #undef MAP_DIFFERENCE_ARGS
     return mllm_check_launch("map_difference");
+}
+
+MLLM_API int mllm_turn_heads(const float* in, int in_stride, void* out, int out_stride, const double* frequencies, int rot_dims, int neighbours, float sign,
+                             const int* positions, int n_rows, int n_heads, int in_size, int out_size, int dtype, hipStream_t stream) {
+    MLLM_REQUIRE(n_rows >= 0 && n_heads > 0 && in_size > 0 && out_size > 0 && out_size <= in_size, "turn_heads: bad sizes");
+    MLLM_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= out_size, "turn_heads: %d turned elements of %d", rot_dims, out_size);
+    MLLM_REQUIRE(in_stride >= n_heads * in_size && out_stride >= n_heads * out_size, "turn_heads: rows are too short for the heads");
+    MLLM_REQUIRE(in != nullptr && out != nullptr && positions != nullptr && (rot_dims == 0 || frequencies != nullptr), "turn_heads: a missing operand");
+    if (n_rows == 0) return 0;
+    const long long items = (long long)n_rows * n_heads;
+    const int blocks = (int)((items + MAP_WAVES - 1) / MAP_WAVES);
+    mllm_count_kernel(MLLM_K_TURN_HEADS);
+#define TURN_HEADS_ARGS(T) in, in_stride, (T*)out, out_stride, frequencies, rot_dims, neighbours, sign, positions, n_rows, n_heads, in_size, out_size
+    if (dtype == MLLM_F32) turn_heads_kernel<float><<<blocks, 64 * MAP_WAVES, 0, stream>>>(TURN_HEADS_ARGS(float));
+    else if (dtype == MLLM_BF16) turn_heads_kernel<bf16_t><<<blocks, 64 * MAP_WAVES, 0, stream>>>(TURN_HEADS_ARGS(bf16_t));
+    else MLLM_REQUIRE(false, "turn_heads: unknown dtype %d", dtype);
+#undef TURN_HEADS_ARGS
+    return mllm_check_launch("turn_heads");
 }

@@ -32,7 +32,8 @@ static const char* const g_kernel_names[MLLM_K_KINDS] = {
     "attention_prefill_stream", "pack", "convert", "decode_attention_half", "decode_mlp_half", "pending_sum",
     "pending_layernorm", "gemm_skinny", "gemm_tiled", "gemm_stream", "static_sum", "probe", "sample", "gemm_best", "choose",
     "rms_norm", "head_norm", "latent_rows", "silu_mul", "heads_linear", "latent_attention", "latent_merge", "projection_rows",
-    "head_gate", "gated_norm", "short_conv", "recurrence", "map_rows", "map_difference",
+    "head_gate", "gated_norm", "short_conv", "recurrence", "map_rows", "map_difference", "turn_heads", "gate_unit", "route",
+    "expert_unit", "branch_join",
 };
 
 void mllm_count_kernel(MllmKernel kind) { g_launches[kind].fetch_add(1, std::memory_order_relaxed); }

@@ -1194,7 +1194,7 @@ def recurrence(q, k, v, state, q_starts, state_slots, n_heads, dim, vdim, *, gat
 
 # -- attention whose heads hold several maps over one value (differential attention) -----------------------------------------
 def map_rows(rows, q_at: int, k_at: int | None, v_at: int | None, q_gain, k_gain, eps, frequencies, rot_dims, positions, slots, k_pages, v_pages,
-             n_heads, n_kv_heads, maps, dim, vdim):
+             n_heads, n_kv_heads, maps, dim, vdim, *, v_frequencies=None, v_rot_dims: int = 0, v_pairing: str = "half"):
     """The row-wise work between the fused projection of a mixer with ``maps`` maps a head and its attention. ``rows``: the float32
     sums of that product, the queries [n_heads, maps, dim] at column ``q_at``, the keys [n_kv_heads, maps, dim] at ``k_at`` and the values
     [n_kv_heads, vdim] at ``v_at`` (both None: the layer reads keys and values another layer keeps, and only its queries are made).
@@ -1203,9 +1203,18 @@ def map_rows(rows, q_at: int, k_at: int | None, v_at: int | None, q_gain, k_gain
     64-bit). Returns the queries as [rows, n_heads * maps * head_size] in the pages' type, laid out for the paged attention kernels run with
     n_heads * maps heads over n_kv_heads * maps key/value heads: query head g R + r (R = n_heads / n_kv_heads) of map m is their head (g *
     maps + m) * R + r. Keys go to head g * maps + m of slots[row] of the pages ([num_pages, n_kv_heads * maps, page_size, head_size]), the
-    value head g to the heads g * maps + 0 .. maps - 1 of the value pages; zeros beyond dim / vdim."""
+    value head g to the heads g * maps + 0 .. maps - 1 of the value pages; zeros beyond dim / vdim.
+    ``v_frequencies`` (float64 [v_rot_dims / 2]; None: values are kept as they are): the first ``v_rot_dims`` elements of every value turn by
+    position * v_frequencies[pair] before they are stored, in pairs (m, m + v_rot_dims / 2) (``v_pairing`` "half") or (2m, 2m + 1)
+    ("neighbours"); whoever attends over such values turns every head's result back by its query's position (``turn_heads``)."""
     num_pages, n_kv, page_size, head_size = k_pages.shape
     _check_pages(k_pages, v_pages, n_kv_heads * maps, head_size)
+    _require(v_pairing in ("half", "neighbours"), "values pair by halves or by neighbours")
+    if v_frequencies is not None and v_rot_dims:
+        _device_tensor(v_frequencies, "v_frequencies", torch.float64, 1)
+        _require(v_rot_dims % 2 == 0 and v_rot_dims <= vdim and v_frequencies.shape[0] >= v_rot_dims // 2, "the values' rotation does not fit them")
+    else:
+        v_frequencies, v_rot_dims = None, 0
     _require(isinstance(rows, torch.Tensor) and rows.is_cuda and rows.dim() == 2 and rows.dtype == torch.float32 and rows.stride(1) == 1,
              "the rows must be float32 GPU rows with contiguous columns")
     n, width = rows.shape
@@ -1231,8 +1240,130 @@ def map_rows(rows, q_at: int, k_at: int | None, v_at: int | None, q_gain, k_gain
     check(library().mllm_map_rows(_ptr(rows), rows.stride(0), int(q_at), int(k_at) if keeps else -1, int(v_at) if keeps else -1, _ptr(q_gain), _ptr(k_gain),
                                   float(eps), _ptr(frequencies if rot_dims else None), int(rot_dims), _ptr(positions), _ptr(slots if keeps else None), _ptr(out),
                                   _ptr(k_pages), _ptr(v_pages), n, n_heads, n_kv_heads, int(maps), dim, vdim, head_size, page_size, _code(k_pages.dtype),
-                                  _stream()))
+                                  _ptr(v_frequencies), int(v_rot_dims), int(v_pairing == "neighbours"), _stream()))
     return out
+
+
+def turn_heads(x, frequencies, rot_dims: int, positions, n_heads: int, in_size: int, out_size: int, *, sign: float = 1.0, pairing: str = "half",
+               out_dtype=None):
+    """Every head of float32 rows x [rows, n_heads * in_size] (rows may be strided) with its first ``rot_dims`` elements turned by sign *
+    position * frequencies[pair] (float64; pairs as in ``map_rows``), the rest copied, out as [rows, n_heads * out_size] of ``out_dtype``
+    (out_size <= in_size: heads kept wider than their values leave at the values' size). sign -1 undoes the turn of sign 1: a head's
+    sum over values that were turned by their own positions, turned back by the query's position, depends on the distances alone."""
+    _rows_f32(x, "x", n_heads * in_size)
+    _require(pairing in ("half", "neighbours"), "pairs go by halves or by neighbours")
+    _require(0 < out_size <= in_size and rot_dims % 2 == 0 and 0 <= rot_dims <= out_size, "the turned elements do not fit the heads")
+    if rot_dims:
+        _device_tensor(frequencies, "frequencies", torch.float64, 1)
+        _require(frequencies.shape[0] >= rot_dims // 2, "fewer frequencies than pairs")
+    n = x.shape[0]
+    _device_tensor(positions, "positions", torch.int32, 1)
+    _require(positions.shape[0] >= n, "fewer positions than rows")
+    out = torch.empty((n, n_heads * out_size), dtype=out_dtype or torch.float32, device=x.device)
+    check(library().mllm_turn_heads(_ptr(x), x.stride(0), _ptr(out), out.stride(0), _ptr(frequencies if rot_dims else None), int(rot_dims),
+                                    int(pairing == "neighbours"), float(sign), _ptr(positions), n, n_heads, in_size, out_size, _code(out.dtype), _stream()))
+    return out
+
+
+# -- layers whose branches run side by side, feed-forwards with clamped gate units, feed-forwards of routed experts ---------------------
+def gate_unit(both, limit: float | None = None, alpha: float = 1.0, shift: float = 0.0):
+    """g * sigmoid(alpha * g) * (u + shift) for rows [gate | up] of a fused gate / up product, g = min(gate, limit), u = clamp(up, -limit,
+    limit) (``limit`` None: unclamped): [rows, 2 * inner] -> [rows, inner]."""
+    _device_tensor(both, "both", dim=2)
+    _require(both.shape[1] % 2 == 0, "the rows do not hold two halves")
+    _require(limit is None or limit > 0, "the limit must be positive")
+    n, inner = both.shape[0], both.shape[1] // 2
+    out = torch.empty((n, inner), dtype=both.dtype, device=both.device)
+    check(library().mllm_gate_unit(_ptr(both), _ptr(out), n, inner, float("inf") if limit is None else float(limit), float(alpha), float(shift),
+                                   _code(both.dtype), _stream()))
+    return out
+
+
+ROUTE_MAX_EXPERTS = 1024
+
+
+def route(logits, n_experts: int, top: int, *, correction=None, n_groups: int = 1, keep: int = 1, floor: float = 0.0):
+    """A router's choice, row by row. ``logits``: float32 rows whose first ``n_experts`` columns are the router's sums (rows may be
+    strided). Scores are their softmax over all experts; the choice goes by score + correction (float32 [n_experts]; None: by the score)
+    among the experts of the ``keep`` best of ``n_groups`` equal groups of neighbours (a group counts by its best choice score); the ``top``
+    best are picked. Returns float32 [rows, n_experts]: a picked expert's score over (the sum of the picked scores + floor), zero for the rest."""
+    _require(isinstance(logits, torch.Tensor) and logits.is_cuda and logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1
+             and logits.shape[1] >= n_experts, "the router's sums must be float32 GPU rows with contiguous columns")
+    _require(1 <= n_experts <= ROUTE_MAX_EXPERTS, f"the router kernel takes up to {ROUTE_MAX_EXPERTS} experts")
+    _require(n_groups >= 1 and n_experts % n_groups == 0 and 1 <= keep <= n_groups, "the experts do not divide into the groups")
+    _require(1 <= top <= keep * (n_experts // n_groups), "more experts to pick than the kept groups hold")
+    if correction is not None:
+        _device_tensor(correction, "correction", torch.float32, 1)
+        _require(correction.shape[0] == n_experts, "one correction an expert")
+    n = logits.shape[0]
+    weights = torch.empty((n, n_experts), dtype=torch.float32, device=logits.device)
+    check(library().mllm_route(_ptr(logits), logits.stride(0), _ptr(correction), _ptr(weights), n_experts, n, n_experts, int(top), int(n_groups), int(keep),
+                               float(floor), _stream()))
+    return weights
+
+
+def expert_unit(up, weights, n_routed: int, ff: int, shared: int = 0, *, h=None, n_identity: int = 0):
+    """Between the up product over all experts' matrices and the down product over all their down matrices: ``up`` [rows, n_routed * ff +
+    shared] -> relu(up)^2 times the row's weight for the unit's expert (``weights``: float32 [rows, >= n_routed + n_identity] as ``route``
+    leaves them; the last ``shared`` units belong to an expert every row uses, weight 1). With ``n_identity`` experts that hand their
+    input on (``h``: the layer's input rows, of up's type) also returns float32 [rows, width], h times the sum of those experts' weights
+    (else None)."""
+    _device_tensor(up, "up", dim=2)
+    n = up.shape[0]
+    _require(up.shape[1] == n_routed * ff + shared, "the hidden units do not match the experts")
+    _require(isinstance(weights, torch.Tensor) and weights.is_cuda and weights.dim() == 2 and weights.dtype == torch.float32 and weights.stride(1) == 1
+             and weights.shape[0] == n and weights.shape[1] >= n_routed + n_identity, "the weights must be float32 GPU rows, one column an expert")
+    carried, width = None, 0
+    if n_identity:
+        _device_tensor(h, "h", up.dtype, 2)
+        _require(h.shape[0] == n, "h and up differ in rows")
+        width = h.shape[1]
+        carried = torch.empty((n, width), dtype=torch.float32, device=up.device)
+    out = torch.empty_like(up)
+    check(library().mllm_expert_unit(_ptr(up), _ptr(out), _ptr(weights), weights.stride(0), n, int(n_routed), int(ff), int(shared), _ptr(h if n_identity else None),
+                                     _ptr(carried), int(n_identity), int(width), _code(up.dtype), _stream()))
+    return out, carried
+
+
+def branch_join(stream, a, b=None, *, a_bias=None, b_bias=None, scale_a=None, scale_b=None, gates=None, gate_a_at: int = 0, gate_b_at: int = 0,
+                mult: float = 1.0, next_weight=None, one_plus: bool = False, eps: float = 0.0, out_dtype=None):
+    """stream + mult * (scale_a * sigmoid(gate_a) * a + scale_b * sigmoid(gate_b) * b), float32 [rows, width]: the sum of a layer whose
+    branches a and b (None: one branch) read the same normed input. a, b: float32 [rows, width] or [n, rows, width], the partial products of
+    a product cut along K, added up here (with ``*_bias``, float32 [width]). ``scale_*``: float32 [width] or None; ``gates``: float32 rows
+    (strided) holding a's gate at column ``gate_a_at`` and b's at ``gate_b_at``, before their sigmoid, or None. With ``next_weight`` (and
+    ``eps``, ``one_plus``, ``out_dtype``) also returns the sum RMS-normed with that gain, in ``out_dtype``: (sum, normed rows)."""
+    _device_tensor(stream, "stream", torch.float32, 2)
+    n, width = stream.shape
+
+    def partials(t, name):
+        if t is None:
+            return None, 0, 0
+        _device_tensor(t, name, torch.float32)
+        _require(t.dim() in (2, 3) and tuple(t.shape[-2:]) == (n, width), f"{name} must have the stream's shape")
+        return t, (t.shape[0] if t.dim() == 3 else 1), (t.stride(0) if t.dim() == 3 else 0)
+
+    a, n_a, a_stride = partials(a, "a")
+    b, n_b, b_stride = partials(b, "b")
+    _require(a is not None, "a layer has at least one branch")
+    for vector, name in ((a_bias, "a_bias"), (b_bias, "b_bias"), (scale_a, "scale_a"), (scale_b, "scale_b"), (next_weight, "next_weight")):
+        if vector is not None:
+            _device_tensor(vector, name, torch.float32, 1)
+            _require(vector.shape[0] == width, f"{name} does not match the row width")
+    gates_stride = 0
+    if gates is not None:
+        _require(gates.is_cuda and gates.dim() == 2 and gates.dtype == torch.float32 and gates.stride(1) == 1 and gates.shape[0] == n, "the gates must be float32 GPU rows")
+        gates_stride = gates.stride(0)
+        _require(0 <= gate_a_at and gate_a_at + width <= gates.shape[1] and (b is None or (0 <= gate_b_at and gate_b_at + width <= gates.shape[1])),
+                 "the gates lie beyond their rows")
+    out = torch.empty((n, width), dtype=torch.float32, device=stream.device)
+    rows = None
+    if next_weight is not None:
+        _require(out_dtype is not None and eps > 0, "a norm behind the sum needs its eps and the rows' type")
+        rows = torch.empty((n, width), dtype=out_dtype, device=stream.device)
+    check(library().mllm_branch_join(_ptr(stream), _ptr(a), n_a, a_stride, _ptr(a_bias), _ptr(b), n_b, b_stride, _ptr(b_bias), _ptr(scale_a), _ptr(scale_b),
+                                     _ptr(gates), gates_stride, int(gate_a_at), int(gate_b_at), float(mult), _ptr(out), _ptr(next_weight), int(bool(one_plus)),
+                                     float(eps), _ptr(rows), 0 if rows is None else _code(rows.dtype), n, width, _stream()))
+    return out if rows is None else (out, rows)
 
 
 def map_difference(maps_out, gate, lam: float, eps: float, n_heads, n_kv_heads, vdim, head_size, scale: float = 1.0, out=None, out_dtype=None):

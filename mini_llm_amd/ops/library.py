@@ -52,7 +52,13 @@ _SIGNATURES = {
     "mllm_latent_rows": [P, c_int, P, c_int, P, c_float, P, c_float, c_int, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_silu_mul": [P, P, c_int, c_int, c_int, P],
     "mllm_map_rows": [P, c_int, c_int, c_int, c_int, P, P, c_float, P, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                      c_int, P],
+                      c_int, P, c_int, c_int, P],
+    "mllm_turn_heads": [P, c_int, P, c_int, P, c_int, c_int, c_float, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_route": [P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, P],
+    "mllm_expert_unit": [P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, c_int, c_int, c_int, P],
+    "mllm_gate_unit": [P, P, c_int, c_int, c_float, c_float, c_float, c_int, P],
+    "mllm_branch_join": [P, P, c_int, c_longlong, P, P, c_int, c_longlong, P, P, P, P, c_int, c_int, c_int, c_float, P, P, c_int, c_float, P, c_int,
+                         c_int, c_int, P],
     "mllm_map_difference": [P, c_int, P, c_int, P, c_int, c_float, c_float, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_heads_linear": [P, c_int, c_int, c_int, P, c_int, P, c_int, c_int, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_latent_attention_supported": [c_int, c_int, c_int],

@@ -145,7 +145,89 @@ class SandwichNormBlock(Block):
         return self._added(self.norm_2b, hidden.stream, self.feed_forward.forward(hidden.rows, None), self._following)
 
 
+class ParallelBlock(Block):
+    """One norm, both branches side by side on its output: with h = norm_1(x), x <- x + mult * (s1 * g1 * mixer(h) + s2 * g2 *
+    feed_forward(h)). ``feed_forward`` None: the layer has its mixer alone. ``layer_scale``: s1, s2 are stored vectors (``ls1``,
+    ``ls2``) that multiply a branch's result element by element (else 1). ``gated``: g1 = sigmoid(W1 h + b1), g2 = sigmoid(W2 h + b2) with
+    stored matrices ``rg1``, ``rg2`` [width, width] and biases ``rg1.b``, ``rg2.b`` (else 1); both gates come from one product over the two
+    matrices laid behind each other, in 32-bit. The sum is one kernel (``kernels.branch_join``: it also adds up the partial products of a
+    branch whose last product was cut along K), which norms the sum for the layer that follows where that layer's first norm is known
+    (``hand_to``): the layer then returns kernels.ReadyRows, and a layer that is handed rows made by its own ``norm_1`` does not run it."""
+
+    takes_pending = True   # takes plain rows, pending rows or the ReadyRows of the layer before
+
+    def __init__(self, norm_1: Norm, mixer: Mixer, feed_forward: FeedForward | None, width: int, compute_dtype, *, mult: float = 1.0,
+                 layer_scale: bool = False, gated: bool = False, names=("norm1", "mix.", "mlp.")):
+        self.norm_1, self.mixer, self.feed_forward = norm_1, mixer, feed_forward
+        self.width, self.compute_dtype, self.mult, self.layer_scale, self.gated = width, compute_dtype, float(mult), bool(layer_scale), bool(gated)
+        self._names = names
+        self._following = None
+        self.scale_1 = self.scale_2 = self.gates = self.gates_bias = None
+
+    def children(self):
+        parts = dict(zip(self._names, (self.norm_1, self.mixer, self.feed_forward)))
+        return {name: part for name, part in parts.items() if part is not None}
+
+    def mixer_part(self):
+        return self.mixer
+
+    def hand_to(self, norm: Norm | None):
+        self._following = norm
+
+    def _branches(self):
+        return ("1", "2") if self.feed_forward is not None else ("1",)
+
+    def tensor_specs(self):
+        from ..weights.spec import TABLE, VECTOR, Normal, TensorSpec
+
+        specs = {}
+        for n in self._branches():
+            if self.layer_scale:
+                specs["ls" + n] = TensorSpec((self.width,), VECTOR, Normal(0.2, mean=1.0))
+            if self.gated:
+                specs["rg" + n] = TensorSpec((self.width, self.width), TABLE, Normal(self.width ** -0.5))
+                specs["rg" + n + ".b"] = TensorSpec((self.width,), VECTOR, Normal(0.5))
+        return specs
+
+    def bind(self, tensors):
+        import torch
+
+        from ..ops import kernels
+        from .linear import fuse_rows
+
+        if self.layer_scale:
+            self.scale_1, self.scale_2 = tensors["ls1"], tensors.get("ls2")
+        if self.gated:
+            fused = fuse_rows([tensors["rg" + n] for n in self._branches()])
+            self.gates = kernels.pack_matrix(fused) if fused.is_cuda else fused
+            self.gates_bias = torch.zeros((fused.shape[0],), dtype=torch.float32, device=fused.device)
+            for index, n in enumerate(self._branches()):
+                self.gates_bias[index * self.width : (index + 1) * self.width] = tensors["rg" + n + ".b"]
+
+    def forward(self, hidden, ctx: LayerContext):
+        import torch
+
+        from ..ops import kernels
+
+        if isinstance(hidden, kernels.ReadyRows) and hidden.norm is self.norm_1:
+            stream, rows = hidden.stream, hidden.rows
+        else:
+            stream = kernels.settle(hidden)
+            rows = self.norm_1.forward(stream, self.compute_dtype)
+        gates = kernels.linear(rows, self.gates, self.gates_bias, out_dtype=torch.float32) if self.gated else None
+        first = self.mixer.forward(rows, None, ctx)
+        second = self.feed_forward.forward(rows, None) if self.feed_forward is not None else None
+        following = self._following
+        ahead = {}
+        if following is not None and hasattr(following, "one_plus") and getattr(following, "out_scale", 1.0) == 1.0:
+            ahead = dict(next_weight=following.weight, one_plus=following.one_plus, eps=following.eps, out_dtype=self.compute_dtype)
+        joined = kernels.branch_join(stream, first, second, scale_a=self.scale_1, scale_b=self.scale_2, gates=gates, gate_a_at=0, gate_b_at=self.width,
+                                     mult=self.mult, **ahead)
+        return kernels.ReadyRows(joined[0], joined[1], following) if ahead else joined
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)
 register_part("block", "sandwich_norm", SandwichNormBlock)
 register_part("block", "post_norm", PostNormBlock)
 register_part("block", "branch_norm", BranchNormBlock)

@@ -76,5 +76,47 @@ class GatedMLP(FeedForward):
         return self._down_product(inner, self.down, residual)
 
 
+class ClampedGatedMLP(FeedForward):
+    """down(g * sigmoid(alpha g) * (u + shift)) with g = min(gate x, limit) and u = clamp(up x, -limit, limit) (``limit`` None:
+    unclamped); with ``biases`` every product has one, stored under the matrix's name + ".b". Gate and up run as one product over the
+    two matrices laid behind each other (biases inside), the gate unit as one kernel over its halves."""
+
+    def __init__(self, width: int, inner: int, limit: float | None, alpha: float = 1.0, shift: float = 0.0, biases: bool = True,
+                 names=("gate", "up", "down")):
+        if limit is not None and not limit > 0:
+            raise ValueError(f"the limit must be positive, not {limit}")
+        self.width, self.inner, self.limit, self.alpha, self.shift, self.biases = width, inner, limit, float(alpha), float(shift), bool(biases)
+        self._names = names
+        self.gate_up = self.gate_up_bias = self.down = self.down_bias = None
+        self._down_product = BranchProduct()
+
+    def tensor_specs(self):
+        from ..weights.spec import MATRIX, TABLE, VECTOR, Normal, TensorSpec
+
+        gate, up, down = self._names
+        specs = {gate: TensorSpec((self.inner, self.width), TABLE, Normal(self.width ** -0.5)),
+                 up: TensorSpec((self.inner, self.width), TABLE, Normal(self.width ** -0.5)),
+                 down: TensorSpec((self.width, self.inner), MATRIX, Normal(self.inner ** -0.5))}
+        if self.biases:
+            specs[gate + ".b"] = TensorSpec((self.inner,), VECTOR, Normal(0.1))
+            specs[up + ".b"] = TensorSpec((self.inner,), VECTOR, Normal(0.1))
+            specs[down + ".b"] = TensorSpec((self.width,), VECTOR, Normal(0.1))
+        return specs
+
+    def bind(self, tensors):
+        gate, up, down = self._names
+        both = torch.cat([tensors[gate], tensors[up]], dim=0).contiguous()
+        self.gate_up = kernels.pack_matrix(both) if both.is_cuda else both
+        self.down = tensors[down]
+        if self.biases:
+            self.gate_up_bias = torch.cat([tensors[gate + ".b"], tensors[up + ".b"]]).contiguous()
+            self.down_bias = tensors[down + ".b"]
+
+    def forward(self, x, residual):
+        inner = kernels.gate_unit(kernels.linear(x, self.gate_up, self.gate_up_bias), self.limit, self.alpha, self.shift)
+        return self._down_product(inner, self.down, residual, bias=self.down_bias)
+
+
 register_part("feed_forward", "dense_mlp", DenseMLP)
+register_part("feed_forward", "clamped_gated_mlp", ClampedGatedMLP)
 register_part("feed_forward", "gated_mlp", GatedMLP)
