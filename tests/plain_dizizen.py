@@ -204,3 +204,89 @@ def forward(config: dict, tensors: dict, tokens, round_to=None, streams: list | 
             streams.append(x.copy())
     x = centred_rms_norm(x, tensors["final.norm"], float(config["norm"]["eps"]))
     return product(x, tensors["head"], rnd)
+
+
+def tensor_shapes(config: dict) -> dict:
+    """name -> shape of every tensor a model of this configuration has."""
+    width, vocab = int(config["width"]), int(config["vocab"])
+    shapes = {"embed": (vocab, width), "final.norm": (width,), "head": (vocab, width)}
+    for index, layer in enumerate(config["layers"]):
+        p, mixer, mlp = f"l{index}.", layer["mixer"], layer.get("mlp")
+        H, G, dim, vdim = (int(mixer[key]) for key in ("heads", "kv_heads", "dim", "vdim"))
+        shapes[p + "norm1"] = (width,)
+        for n in ("1", "2") if mlp is not None else ("1",):
+            shapes.update({p + "ls" + n: (width,), p + "rg" + n: (width, width), p + "rg" + n + ".b": (width,)})
+        shapes.update({p + "mix.q": (H * dim, width), p + "mix.q.b": (H * dim,), p + "mix.o": (width, H * vdim), p + "mix.o.b": (width,)})
+        if mixer.get("kv_from") is None:
+            shapes.update({p + "mix.k": (G * dim, width), p + "mix.k.b": (G * dim,), p + "mix.v": (G * vdim, width), p + "mix.v.b": (G * vdim,)})
+        if mlp is None:
+            continue
+        if mlp["kind"] == "dense":
+            ff = int(mlp["ff"])
+            shapes.update({p + "mlp.gate": (ff, width), p + "mlp.gate.b": (ff,), p + "mlp.up": (ff, width), p + "mlp.up.b": (ff,),
+                           p + "mlp.down": (width, ff), p + "mlp.down.b": (width,)})
+        else:
+            router = mlp["router"]
+            outputs = int(router["experts"]) + int(router.get("identity", 0))
+            shapes.update({p + "mlp.router": (outputs, width), p + "mlp.correction": (outputs,)})
+            ff = int(mlp["expert"]["ff"])
+            for e in range(int(router["experts"])):
+                shapes.update({p + f"mlp.e{e}.up": (ff, width), p + f"mlp.e{e}.down": (width, ff)})
+            if mlp.get("shared"):
+                ff = int(mlp["shared"]["ff"])
+                shapes.update({p + "mlp.shared.up": (ff, width), p + "mlp.shared.down": (width, ff)})
+    return shapes
+
+
+def greedy(config: dict, tensors: dict, prompt, n_new: int, round_to=None) -> list:
+    tokens = list(prompt)
+    for _ in range(n_new):
+        tokens.append(int(forward(config, tensors, tokens, round_to)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+# -- random models for the tests ------------------------------------------------------------------------------------------
+def random_weights(config: dict, seed: int) -> dict:
+    """Weights whose activations stay of order one and whose every mechanism moves the logits: matrices ~ N(0, 1/in) (the router's
+    larger, so that its scores differ), norm gains around zero, layer scales around one, biases of order one, corrections of the size
+    of the scores. The embedding is drawn so that its rows times embedding.scale are of order one. float32 arrays holding bfloat16
+    values (as files hold them)."""
+    import plain_gpt2
+
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shape in tensor_shapes(config).items():
+        last = name.rsplit(".", 1)[-1]
+        if last in ("norm", "norm1"):
+            value = rng.normal(0.0, 0.1, shape)
+        elif last in ("ls1", "ls2"):
+            value = rng.normal(1.0, 0.3, shape)
+        elif last == "correction":
+            value = rng.normal(0.0, 0.5 / shape[0], shape)
+        elif last == "b":
+            value = rng.normal(0.0, 0.3, shape)
+        elif name == "embed":
+            value = rng.normal(0.0, 1.0 / float(config["embedding"]["scale"]), shape)
+        elif last == "router":
+            value = rng.normal(0.0, 2.0 * shape[1] ** -0.5, shape)
+        else:
+            value = rng.normal(0.0, shape[1] ** -0.5, shape)
+        out[name] = plain_gpt2.round_to_bf16(np.asarray(value, dtype=np.float32))
+    return out
+
+
+def as_float64(weights: dict) -> dict:
+    return {name: np.asarray(value, dtype=np.float64) for name, value in weights.items()}
+
+
+def write_model_dir(path, config: dict, weights: dict):
+    import json
+    from pathlib import Path
+
+    import plain_gpt2
+
+    path = Path(path)
+    path.mkdir(parents=True, exist_ok=True)
+    (path / "config.json").write_text(json.dumps(config, indent=1))
+    plain_gpt2.write_safetensors(path / "model.safetensors", {k: np.asarray(v, dtype=np.float32) for k, v in weights.items()}, bf16=True)
+    return path
