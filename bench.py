@@ -340,7 +340,8 @@ _KERNEL_CLASSES = {
     "products": ("gemm", "gemm_split", "gemm_qkv_cache", "gemm_best", "heads_linear"),
     "attention": ("attention", "attention_decode", "attention_prefill", "latent_attention"),
     "row-wise": ("layernorm", "pending_layernorm", "rms_norm", "head_norm", "latent_rows", "silu_mul", "pending_sum", "add", "cache_write", "embed",
-                 "projection_rows", "head_gate", "gated_norm", "short_conv", "map_rows", "map_difference"),
+                 "projection_rows", "head_gate", "gated_norm", "short_conv", "map_rows", "map_difference", "turn_heads", "gate_unit", "route", "expert_unit",
+                 "branch_join"),
     "recurrence": ("recurrence",),
     "layer kernels": ("decode_attention_half", "decode_mlp_half"),
     "choice": ("choose", "sample"),
@@ -410,9 +411,27 @@ def perezen_shape(width: int, layers: int, vocab: int = 50257) -> dict:
     return {"architecture": "Perezen", "vocab": vocab, "width": width, "max_positions": CONTEXT, "norm": {"eps": 1e-5}, "logit_scale": 1.0, "layers": out}
 
 
+def dizizen_shape(width: int, layers: int, vocab: int = 50257) -> dict:
+    """Layers in fours, all attention (heads of 64, a key/value head for every four, queries, keys and values rotated), the third reading
+    the keys and values the second keeps; the first and third with a dense feed-forward of 8/3 x width (a clamped gate unit), the second
+    and fourth with routed experts: six experts of 1 x width and two that hand their input on, in two groups of which one is kept, two
+    picked, and a shared expert of 2 x width (as many multiply-adds a token as the dense feed-forward, for the picked experts)."""
+    heads = width // 64
+    ff = -(-(8 * width // 3) // 64) * 64
+    mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 64, "vdim": 64, "scale": 0.125, "rot": {"dims": 64, "base": 10000.0}}
+    dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+    routed = {"kind": "moe", "expert": {"ff": width}, "shared": {"ff": 2 * width},
+              "router": {"experts": 6, "identity": 2, "top": 2, "groups": {"count": 2, "keep": 1}}}
+    out = []
+    for index in range(layers):
+        out.append({"type": "attention", "mixer": dict(mixer, kv_from=index - 1) if index % 4 == 2 else mixer, "mlp": routed if index % 2 else dense})
+    return {"architecture": "Dizizen", "vocab": vocab, "width": width, "embedding": {"scale": width ** 0.5}, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+            "layers": out}
+
+
 def measure_design(args) -> dict:
     """Prefill and decode throughput of a design and of the framework's closest older model with as many layers of the same width
-    (random weights): Gimozen beside GPT-2, Ketolix beside Gimozen, Perezen beside Ketolix; and where each model's step spends its time, by class of
+    (random weights): Gimozen beside GPT-2, Ketolix beside Gimozen, Perezen beside Ketolix, Dizizen beside Gimozen; and where each model's step spends its time, by class of
     kernel, inside a prompt step and a decode step."""
     import numpy as np
     import torch
@@ -422,7 +441,9 @@ def measure_design(args) -> dict:
     from mini_llm_amd.engine.engine import Engine, EngineOptions
 
     width, layers = DESIGN_SIZES[args.shape]
-    if args.design == "perezen":
+    if args.design == "dizizen":
+        raws = {"dizizen": dizizen_shape(width, layers), "gimozen": gimozen_shape(width, layers)}
+    elif args.design == "perezen":
         raws = {"perezen": perezen_shape(width, layers), "ketolix": ketolix_shape(width, layers)}
     elif args.design == "ketolix":
         raws = {"ketolix": ketolix_shape(width, layers), "gimozen": gimozen_shape(width, layers)}
@@ -689,8 +710,8 @@ def main() -> int:
     parser.add_argument("--serving", action="store_true", help="continuous batching of 64 requests on the GPT-2 medium shape through the scheduler")
     parser.add_argument("--temperature", type=float, default=0.0, help="sampling temperature of --serving (0: greedy)")
     parser.add_argument("--step-by-step", action="store_true", help="--serving reads every step's tokens before it launches the next")
-    parser.add_argument("--design", default=None, choices=("gimozen", "ketolix", "perezen"), help="a design beside the closest older model with as many layers of the same width "
-                        "(--shape small|medium): Gimozen beside GPT-2, Ketolix beside Gimozen, Perezen beside Ketolix; prefill and decode throughput of both, and where their steps spend the time")
+    parser.add_argument("--design", default=None, choices=("gimozen", "ketolix", "perezen", "dizizen"), help="a design beside the closest older model with as many layers of the same width "
+                        "(--shape small|medium): Gimozen beside GPT-2, Ketolix beside Gimozen, Perezen beside Ketolix, Dizizen beside Gimozen; prefill and decode throughput of both, and where their steps spend the time")
     parser.add_argument("--peaks", action="store_true", help="measure this machine's read bandwidth and matrix-core rate with the library's probes")
     args = parser.parse_args()
     if args.gpus != 1:

@@ -71,38 +71,103 @@ __global__ __launch_bounds__(WAVE) void route_kernel(const float* __restrict__ l
 }
 
 // up: [rows, n_routed * ff + shared] hidden units before their activation, expert by expert, then `shared` units of an expert that
-// every row uses. out = relu(up)^2 * weights[row, expert] (shared units: relu(up)^2). Behind the hidden units the grid goes on over
-// `width` columns of `carried` (null: none): carried[row, :] = h[row, :] * (the sum of weights[row, n_routed .. n_routed + n_identity)),
-// the share of the experts that hand their input on as it is.
-template <typename T>
+// every row uses. out = relu(up)^2 * weights[row, expert] (shared units: relu(up)^2). Behind the `unit_blocks` blocks of the hidden units
+// the grid goes on over `width` columns of `carried` (null: none): carried[row, :] = h[row, :] * (the sum of weights[row, n_routed ..
+// n_routed + n_identity)), the share of the experts that hand their input on as it is. PIECES: a thread takes 16 bytes of units (ff and
+// shared are multiples of that many units, so a piece lies in one expert).
+template <typename T, bool PIECES>
 __global__ __launch_bounds__(256) void expert_unit_kernel(const T* __restrict__ up, T* __restrict__ out, const float* __restrict__ weights, int weights_stride,
                                                           int n_routed, int ff, int shared, const T* __restrict__ h, float* __restrict__ carried,
-                                                          int n_identity, int width) {
+                                                          int n_identity, int width, int unit_blocks) {
+    constexpr int VEC = PIECES ? 16 / (int)sizeof(T) : 1;
     const int inner = n_routed * ff + shared;
-    const int j = blockIdx.x * blockDim.x + threadIdx.x;
     const size_t row = blockIdx.y;
     const float* w = weights + row * weights_stride;
-    if (j < inner) {
-        const float u = fmaxf(to_float(up[row * inner + j]), 0.0f);
-        const float weight = j < n_routed * ff ? w[j / ff] : 1.0f;
-        out[row * inner + j] = from_float<T>(u * u * weight);
-    } else if (carried != nullptr && j - inner < width) {
+    if ((int)blockIdx.x >= unit_blocks) {
+        const int j = ((int)blockIdx.x - unit_blocks) * blockDim.x + threadIdx.x;
+        if (carried == nullptr || j >= width) return;
         float share = 0.0f;
         for (int e = 0; e < n_identity; e++) share += w[n_routed + e];
-        carried[row * width + (j - inner)] = to_float(h[row * width + (j - inner)]) * share;
+        carried[row * width + j] = to_float(h[row * width + j]) * share;
+        return;
+    }
+    const int j = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+    if (j >= inner) return;
+    const float weight = j < n_routed * ff ? w[j / ff] : 1.0f;
+    if constexpr (PIECES) {
+        const Vec16 in = *reinterpret_cast<const Vec16*>(up + row * inner + j);
+        Vec16 result;
+        const T* ie = reinterpret_cast<const T*>(&in);
+        T* re = reinterpret_cast<T*>(&result);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            const float u = fmaxf(to_float(ie[e]), 0.0f);
+            re[e] = from_float<T>(u * u * weight);
+        }
+        *reinterpret_cast<Vec16*>(out + row * inner + j) = result;
+    } else {
+        const float u = fmaxf(to_float(up[row * inner + j]), 0.0f);
+        out[row * inner + j] = from_float<T>(u * u * weight);
     }
 }
 
 // both: [rows, 2 * inner], a gate half and an up half. out = g * sigmoid(alpha * g) * (u + shift) with g = min(gate, limit) and u =
-// clamp(up, -limit, limit) (limit infinite: unclamped).
-template <typename T>
+// clamp(up, -limit, limit) (limit infinite: unclamped). PIECES: a thread takes 16 bytes of each half.
+template <typename T, bool PIECES>
 __global__ __launch_bounds__(256) void gate_unit_kernel(const T* __restrict__ both, T* __restrict__ out, int inner, float limit, float alpha, float shift) {
-    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    constexpr int VEC = PIECES ? 16 / (int)sizeof(T) : 1;
+    const int j = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     if (j >= inner) return;
     const size_t row = blockIdx.y;
-    const float g = fminf(to_float(both[row * 2 * inner + j]), limit);
-    const float u = fminf(fmaxf(to_float(both[row * 2 * inner + inner + j]), -limit), limit);
-    out[row * inner + j] = from_float<T>(g / (1.0f + expf(-alpha * g)) * (u + shift));
+    const T* g_at = both + row * 2 * inner + j;
+    const T* u_at = g_at + inner;
+    T* out_at = out + row * inner + j;
+    if constexpr (PIECES) {
+        const Vec16 gs = *reinterpret_cast<const Vec16*>(g_at), us = *reinterpret_cast<const Vec16*>(u_at);
+        Vec16 result;
+        const T* ge = reinterpret_cast<const T*>(&gs);
+        const T* ue = reinterpret_cast<const T*>(&us);
+        T* re = reinterpret_cast<T*>(&result);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            const float g = fminf(to_float(ge[e]), limit);
+            const float u = fminf(fmaxf(to_float(ue[e]), -limit), limit);
+            re[e] = from_float<T>(g / (1.0f + expf(-alpha * g)) * (u + shift));
+        }
+        *reinterpret_cast<Vec16*>(out_at) = result;
+    } else {
+        const float g = fminf(to_float(*g_at), limit);
+        const float u = fminf(fmaxf(to_float(*u_at), -limit), limit);
+        *out_at = from_float<T>(g / (1.0f + expf(-alpha * g)) * (u + shift));
+    }
+}
+
+template <typename T>
+void launch_expert_unit(const void* up, void* out, const float* weights, int weights_stride, int rows, int n_routed, int ff, int shared, const void* h,
+                        float* carried, int n_identity, int width, hipStream_t stream) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    const int inner = n_routed * ff + shared;
+    const bool pieces = ff % VEC == 0 && shared % VEC == 0 && ((uintptr_t)up & 15) == 0 && ((uintptr_t)out & 15) == 0;
+    const int unit_blocks = ceil_div(pieces ? inner / VEC : inner, 256);
+    dim3 grid(unit_blocks + (carried != nullptr ? ceil_div(width, 256) : 0), rows);
+    if (pieces)
+        expert_unit_kernel<T, true><<<grid, 256, 0, stream>>>((const T*)up, (T*)out, weights, weights_stride, n_routed, ff, shared, (const T*)h, carried, n_identity,
+                                                              width, unit_blocks);
+    else
+        expert_unit_kernel<T, false><<<grid, 256, 0, stream>>>((const T*)up, (T*)out, weights, weights_stride, n_routed, ff, shared, (const T*)h, carried, n_identity,
+                                                               width, unit_blocks);
+}
+
+template <typename T>
+void launch_gate_unit(const void* both, void* out, int rows, int inner, float limit, float alpha, float shift, hipStream_t stream) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    if (inner % VEC == 0 && ((uintptr_t)both & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+        dim3 grid(ceil_div(inner / VEC, 256), rows);
+        gate_unit_kernel<T, true><<<grid, 256, 0, stream>>>((const T*)both, (T*)out, inner, limit, alpha, shift);
+    } else {
+        dim3 grid(ceil_div(inner, 256), rows);
+        gate_unit_kernel<T, false><<<grid, 256, 0, stream>>>((const T*)both, (T*)out, inner, limit, alpha, shift);
+    }
 }
 
 }  // namespace
@@ -128,22 +193,16 @@ MLLM_API int mllm_expert_unit(const void* up, void* out, const float* weights, i
     if (n_rows == 0) return 0;
     mllm_count_kernel(MLLM_K_EXPERT_UNIT);
     const long long inner = (long long)n_routed * ff + shared;
-    const int columns = (int)inner + (carried != nullptr ? width : 0);
     const size_t element = dtype == MLLM_F32 ? 4 : 2;
     for (int row0 = 0; row0 < n_rows; row0 += 65535) {   // the grid's second dimension holds 65,535 rows
         const int rows = n_rows - row0 < 65535 ? n_rows - row0 : 65535;
-        dim3 grid(ceil_div(columns, 256), rows);
         const char* up_at = (const char*)up + (size_t)row0 * inner * element;
         char* out_at = (char*)out + (size_t)row0 * inner * element;
         const char* h_at = h == nullptr ? nullptr : (const char*)h + (size_t)row0 * width * element;
         float* carried_at = carried == nullptr ? nullptr : carried + (size_t)row0 * width;
         const float* weights_at = weights + (size_t)row0 * weights_stride;
-        if (dtype == MLLM_F32)
-            expert_unit_kernel<float><<<grid, 256, 0, stream>>>((const float*)up_at, (float*)out_at, weights_at, weights_stride, n_routed, ff, shared,
-                                                                (const float*)h_at, carried_at, n_identity, width);
-        else
-            expert_unit_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)up_at, (bf16_t*)out_at, weights_at, weights_stride, n_routed, ff, shared,
-                                                                 (const bf16_t*)h_at, carried_at, n_identity, width);
+        if (dtype == MLLM_F32) launch_expert_unit<float>(up_at, out_at, weights_at, weights_stride, rows, n_routed, ff, shared, h_at, carried_at, n_identity, width, stream);
+        else launch_expert_unit<bf16_t>(up_at, out_at, weights_at, weights_stride, rows, n_routed, ff, shared, h_at, carried_at, n_identity, width, stream);
     }
     return mllm_check_launch("expert_unit");
 }
@@ -157,11 +216,10 @@ MLLM_API int mllm_gate_unit(const void* both, void* out, int n_rows, int inner, 
     const size_t element = dtype == MLLM_F32 ? 4 : 2;
     for (int row0 = 0; row0 < n_rows; row0 += 65535) {
         const int rows = n_rows - row0 < 65535 ? n_rows - row0 : 65535;
-        dim3 grid(ceil_div(inner, 256), rows);
         const char* in_at = (const char*)both + (size_t)row0 * 2 * inner * element;
         char* out_at = (char*)out + (size_t)row0 * inner * element;
-        if (dtype == MLLM_F32) gate_unit_kernel<float><<<grid, 256, 0, stream>>>((const float*)in_at, (float*)out_at, inner, limit, alpha, shift);
-        else gate_unit_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)in_at, (bf16_t*)out_at, inner, limit, alpha, shift);
+        if (dtype == MLLM_F32) launch_gate_unit<float>(in_at, out_at, rows, inner, limit, alpha, shift, stream);
+        else launch_gate_unit<bf16_t>(in_at, out_at, rows, inner, limit, alpha, shift, stream);
     }
     return mllm_check_launch("gate_unit");
 }
