@@ -54,6 +54,43 @@ __global__ __launch_bounds__(64 * MAP_WAVES) void turn_heads_kernel(const float*
         to[d] = from_float<T>(d < rot_dims ? turned_element(from, d, rot_dims, neighbours, position, frequencies, sign) : from[d]);
 }
 
+// turn_heads_kernel four neighbouring elements a thread (pairing of halves; turned elements, heads and strides in whole fours, rows on 16 bytes).
+template <typename T>
+__global__ __launch_bounds__(256) void turn_heads_pieces_kernel(const float* __restrict__ in, int in_stride, T* __restrict__ out, int out_stride,
+                                                                const double* __restrict__ frequencies, int rot_dims, float sign,
+                                                                const int* __restrict__ positions, int n_rows, int n_heads, int in_size, int out_size) {
+    const int quads = out_size / 4;
+    const long long index = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= (long long)n_rows * n_heads * quads) return;
+    const int row = (int)(index / (n_heads * quads)), within = (int)(index % (n_heads * quads));
+    const int head = within / quads, d = (within % quads) * 4;
+    const float* from = in + (size_t)row * in_stride + (size_t)head * in_size;
+    f32x4 made = *reinterpret_cast<const f32x4*>(from + d);
+    if (d < rot_dims) {
+        const int half = rot_dims / 2;
+        const bool first = d < half;
+        const int pair = first ? d : d - half;
+        const f32x4 partner = *reinterpret_cast<const f32x4*>(from + (first ? d + half : d - half));
+        const int position = positions[row];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float a, b;
+            if (first) turned(made[e], partner[e], position, sign * frequencies[pair + e], a, b);
+            else turned(partner[e], made[e], position, sign * frequencies[pair + e], b, a);
+            made[e] = a;
+        }
+    }
+    T* to = out + (size_t)row * out_stride + (size_t)head * out_size + d;
+    if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<f32x4*>(to) = made;
+    } else {
+        bf16x4 narrow;
+#pragma unroll
+        for (int e = 0; e < 4; e++) narrow[e] = from_float<T>(made[e]);
+        *reinterpret_cast<bf16x4*>(to) = narrow;
+    }
+}
+
 // A wave per (row, item); a row's items are its n_heads * maps queries, then (where the layer keeps keys and values of its own: k_at
 // >= 0) its n_kv_heads * maps keys and its n_kv_heads values. `rows` are the 32-bit sums of the product that made them, [.. | q | k |
 // v | ..] at columns q_at, k_at, v_at: q as [n_heads, maps, dim], k as [n_kv_heads, maps, dim], v as [n_kv_heads, vdim].
@@ -132,6 +169,73 @@ __global__ __launch_bounds__(64 * MAP_WAVES) void map_rows_kernel(
     }
 }
 
+// The same work as map_rows_kernel for heads of one map without a norm, four neighbouring elements a thread: a thread makes elements d ..
+// d + 3 of one query, key or value head from 16 bytes of the head and, where they turn, 16 bytes of their partners (pairing of halves; the
+// turned elements, the elements behind them and the heads themselves come in whole fours, and the rows start on 16 bytes). A wave so makes
+// 256 elements, not 64, and a row's heads need an eighth of the waves.
+template <typename T>
+__global__ __launch_bounds__(256) void rotate_rows_pieces_kernel(
+    const float* __restrict__ rows, int stride, int q_at, int k_at, int v_at, const double* __restrict__ frequencies, int rot_dims,
+    const int* __restrict__ positions, const int* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
+    int n_rows, int n_heads, int n_kv_heads, int dim, int vdim, int head_size, int page_size, const double* __restrict__ v_frequencies, int v_rot_dims) {
+    const int quads = head_size / 4;
+    const int n_kept = k_at >= 0 ? n_kv_heads : 0;
+    const int per_row = (n_heads + 2 * n_kept) * quads;
+    const long long index = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= (long long)n_rows * per_row) return;
+    const int row = (int)(index / per_row), within = (int)(index % per_row);
+    const int item = within / quads, d = (within % quads) * 4;
+    const float* in_row = rows + (size_t)row * stride;
+    const float* in;
+    T* out;
+    int size = dim, turned_dims = rot_dims;
+    const double* f = frequencies;
+    if (item < n_heads) {
+        in = in_row + q_at + (size_t)item * dim;
+        out = q_out + ((size_t)row * n_heads + item) * head_size;
+    } else {
+        const int slot = slots[row];
+        if (slot < 0) return;
+        const bool is_key = item < n_heads + n_kept;
+        const int g = item - n_heads - (is_key ? 0 : n_kept);
+        const size_t place = (((size_t)(slot / page_size) * n_kept + g) * page_size + slot % page_size) * head_size;
+        if (is_key) {
+            in = in_row + k_at + (size_t)g * dim;
+            out = k_pages + place;
+        } else {
+            in = in_row + v_at + (size_t)g * vdim;
+            out = v_pages + place;
+            size = vdim, turned_dims = v_frequencies ? v_rot_dims : 0, f = v_frequencies;
+        }
+    }
+    f32x4 made = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (d < size) {
+        made = *reinterpret_cast<const f32x4*>(in + d);
+        if (d < turned_dims) {
+            const int half = turned_dims / 2;
+            const bool first = d < half;
+            const int pair = first ? d : d - half;
+            const f32x4 partner = *reinterpret_cast<const f32x4*>(in + (first ? d + half : d - half));
+            const int position = positions[row];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float a, b;
+                if (first) turned(made[e], partner[e], position, f[pair + e], a, b);
+                else turned(partner[e], made[e], position, f[pair + e], b, a);
+                made[e] = a;
+            }
+        }
+    }
+    if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<f32x4*>(out + d) = made;
+    } else {
+        bf16x4 narrow;
+#pragma unroll
+        for (int e = 0; e < 4; e++) narrow[e] = from_float<T>(made[e]);
+        *reinterpret_cast<bf16x4*>(out + d) = narrow;
+    }
+}
+
 // A wave per (row, head): with a1 and a2 the results of the head's two maps (attention heads (g * 2 + 0) * R + r and (g * 2 + 1) * R + r
 // of `maps_out`, heads of head_size of which the first vdim count), x = a1 - lambda a2, out = x / sqrt(mean(x^2) + eps) * scale *
 // sigmoid(gate) -> out [row, head * vdim ..]. gate: 32-bit rows (null: no gate), the head's vdim elements at column head * vdim. The
@@ -186,6 +290,22 @@ MLLM_API int mllm_map_rows(const float* rows, int stride, int q_at, int k_at, in
     const long long items = (long long)n_rows * (n_heads * maps + (k_at >= 0 ? n_kv_heads * (maps + 1) : 0));
     const int blocks = (int)((items + MAP_WAVES - 1) / MAP_WAVES);
     mllm_count_kernel(MLLM_K_MAP_ROWS);
+    // one map a head and no norm, everything in whole fours: four elements a thread
+    const bool values_fit = v_frequencies == nullptr || v_rot_dims == 0 || (v_neighbours == 0 && v_rot_dims % 8 == 0);
+    if (maps == 1 && q_gain == nullptr && k_gain == nullptr && rot_dims % 8 == 0 && dim % 4 == 0 && vdim % 4 == 0 && head_size % 4 == 0 && stride % 4 == 0 &&
+        q_at % 4 == 0 && (k_at < 0 || (k_at % 4 == 0 && v_at % 4 == 0)) && ((uintptr_t)rows & 15) == 0 && ((uintptr_t)q_out & 15) == 0 &&
+        (k_at < 0 || (((uintptr_t)k_pages & 15) == 0 && ((uintptr_t)v_pages & 15) == 0)) && values_fit) {
+        const long long threads = (long long)n_rows * (n_heads + (k_at >= 0 ? 2 * n_kv_heads : 0)) * (head_size / 4);
+        const int piece_blocks = (int)((threads + 255) / 256);
+        const double* vf = v_rot_dims > 0 ? v_frequencies : nullptr;
+#define ROTATE_ROWS_ARGS(T) rows, stride, q_at, k_at, v_at, frequencies, rot_dims, positions, slots, (T*)q_out, (T*)k_pages, (T*)v_pages, n_rows, n_heads, \
+                            n_kv_heads, dim, vdim, head_size, page_size, vf, v_rot_dims
+        if (dtype == MLLM_F32) rotate_rows_pieces_kernel<float><<<piece_blocks, 256, 0, stream>>>(ROTATE_ROWS_ARGS(float));
+        else if (dtype == MLLM_BF16) rotate_rows_pieces_kernel<bf16_t><<<piece_blocks, 256, 0, stream>>>(ROTATE_ROWS_ARGS(bf16_t));
+        else MLLM_REQUIRE(false, "map_rows: unknown dtype %d", dtype);
+#undef ROTATE_ROWS_ARGS
+        return mllm_check_launch("map_rows");
+    }
 #define MAP_ROWS_ARGS(T) rows, stride, q_at, k_at, v_at, q_gain, k_gain, eps, frequencies, rot_dims, positions, slots, (T*)q_out, (T*)k_pages, \
                          (T*)v_pages, n_rows, n_heads, n_kv_heads, maps, dim, vdim, head_size, page_size, v_frequencies, v_rot_dims, v_neighbours
     if (dtype == MLLM_F32) map_rows_kernel<float><<<blocks, 64 * MAP_WAVES, 0, stream>>>(MAP_ROWS_ARGS(float));
@@ -228,6 +348,17 @@ MLLM_API int mllm_turn_heads(const float* in, int in_stride, void* out, int out_
     const long long items = (long long)n_rows * n_heads;
     const int blocks = (int)((items + MAP_WAVES - 1) / MAP_WAVES);
     mllm_count_kernel(MLLM_K_TURN_HEADS);
+    if (neighbours == 0 && rot_dims % 8 == 0 && in_size % 4 == 0 && out_size % 4 == 0 && in_stride % 4 == 0 && out_stride % 4 == 0 && ((uintptr_t)in & 15) == 0 &&
+        ((uintptr_t)out & 15) == 0) {
+        const long long threads = items * (out_size / 4);
+        const int piece_blocks = (int)((threads + 255) / 256);
+        if (dtype == MLLM_F32)
+            turn_heads_pieces_kernel<float><<<piece_blocks, 256, 0, stream>>>(in, in_stride, (float*)out, out_stride, frequencies, rot_dims, sign, positions, n_rows, n_heads, in_size, out_size);
+        else if (dtype == MLLM_BF16)
+            turn_heads_pieces_kernel<bf16_t><<<piece_blocks, 256, 0, stream>>>(in, in_stride, (bf16_t*)out, out_stride, frequencies, rot_dims, sign, positions, n_rows, n_heads, in_size, out_size);
+        else MLLM_REQUIRE(false, "turn_heads: unknown dtype %d", dtype);
+        return mllm_check_launch("turn_heads");
+    }
 #define TURN_HEADS_ARGS(T) in, in_stride, (T*)out, out_stride, frequencies, rot_dims, neighbours, sign, positions, n_rows, n_heads, in_size, out_size
     if (dtype == MLLM_F32) turn_heads_kernel<float><<<blocks, 64 * MAP_WAVES, 0, stream>>>(TURN_HEADS_ARGS(float));
     else if (dtype == MLLM_BF16) turn_heads_kernel<bf16_t><<<blocks, 64 * MAP_WAVES, 0, stream>>>(TURN_HEADS_ARGS(bf16_t));

@@ -150,7 +150,7 @@ class ParallelBlock(Block):
     feed_forward(h)). ``feed_forward`` None: the layer has its mixer alone. ``layer_scale``: s1, s2 are stored vectors (``ls1``,
     ``ls2``) that multiply a branch's result element by element (else 1). ``gated``: g1 = sigmoid(W1 h + b1), g2 = sigmoid(W2 h + b2) with
     stored matrices ``rg1``, ``rg2`` [width, width] and biases ``rg1.b``, ``rg2.b`` (else 1); both gates come from one product over the two
-    matrices laid behind each other, in 32-bit. The sum is one kernel (``kernels.branch_join``: it also adds up the partial products of a
+    matrices laid behind each other, in 32-bit: the mixer's own first product where it can carry them (``Mixer.carries_rows``). The sum is one kernel (``kernels.branch_join``: it also adds up the partial products of a
     branch whose last product was cut along K), which norms the sum for the layer that follows where that layer's first norm is known
     (``hand_to``): the layer then returns kernels.ReadyRows, and a layer that is handed rows made by its own ``norm_1`` does not run it."""
 
@@ -199,10 +199,14 @@ class ParallelBlock(Block):
             self.scale_1, self.scale_2 = tensors["ls1"], tensors.get("ls2")
         if self.gated:
             fused = fuse_rows([tensors["rg" + n] for n in self._branches()])
-            self.gates = kernels.pack_matrix(fused) if fused.is_cuda else fused
             self.gates_bias = torch.zeros((fused.shape[0],), dtype=torch.float32, device=fused.device)
             for index, n in enumerate(self._branches()):
                 self.gates_bias[index * self.width : (index + 1) * self.width] = tensors["rg" + n + ".b"]
+            if self.mixer.carries_rows:   # the gates ride along in the mixer's own first product (this part is bound before its children)
+                self.mixer.carry_rows(fused, self.gates_bias)
+                self.gates = None
+            else:
+                self.gates = kernels.pack_matrix(fused) if fused.is_cuda else fused
 
     def forward(self, hidden, ctx: LayerContext):
         import torch
@@ -214,8 +218,10 @@ class ParallelBlock(Block):
         else:
             stream = kernels.settle(hidden)
             rows = self.norm_1.forward(stream, self.compute_dtype)
-        gates = kernels.linear(rows, self.gates, self.gates_bias, out_dtype=torch.float32) if self.gated else None
+        gates = kernels.linear(rows, self.gates, self.gates_bias, out_dtype=torch.float32) if self.gated and self.gates is not None else None
         first = self.mixer.forward(rows, None, ctx)
+        if self.gated and self.gates is None:
+            gates = ctx.extra.pop("carried")
         second = self.feed_forward.forward(rows, None) if self.feed_forward is not None else None
         following = self._following
         ahead = {}

@@ -10,7 +10,7 @@ bias) maps the heads laid behind each other back to the width.
 ``own_keys`` False: the layer has no key and value tensors and reads the pages another layer call keeps (the model's schedule names
 it): that layer's keys after their rotation and its turned values, with queries of its own.
 
-One product makes everything that reads h ([q | k | v], 32-bit sums, biases inside); ``kernels.map_rows`` (a head holding one map, no
+One product makes everything that reads h ([q | k | v], 32-bit sums, biases inside; ``carry_rows`` lays a block's own matrix behind them); ``kernels.map_rows`` (a head holding one map, no
 norm) rotates and writes the pages; the framework's paged attention kernels do the rest, leaving the heads' sums in 32-bit where they
 are turned back (``kernels.turn_heads``) before they are rounded for the output product. Heads of different key and value sizes are kept
 in pages of the larger size (rounded to 16) with zeros behind."""
@@ -30,6 +30,7 @@ from .positions import RotaryEncoding
 class RotaryAttention(Mixer):
     graph_safe = True
     short_portion = kernels.DECODE_MAX_Q_LEN
+    carries_rows = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, dim: int, vdim: int, scale: float, *, rotary: RotaryEncoding | None = None,
                  value_rotary: RotaryEncoding | None = None, biases: bool = True, own_keys: bool = True):
@@ -48,6 +49,13 @@ class RotaryAttention(Mixer):
         self.q_width, self.k_width, self.v_width, self.o_width = n_heads * dim, n_kv_heads * dim, n_kv_heads * vdim, n_heads * vdim
         self.w_in = self.b_in = self.o = self.o_bias = None
         self._out_product = BranchProduct()
+        self._carried = None      # (matrix, bias) of rows that ride along in the input product, and where their columns start
+        self._carried_at = 0
+
+    def carry_rows(self, matrix, bias=None):
+        if matrix.dim() != 2 or matrix.shape[1] != self.width:
+            raise ValueError(f"rows that ride along read the same {self.width} inputs")
+        self._carried = (matrix, bias)
 
     def _input_names(self):
         return ("q", "k", "v") if self.own_keys else ("q",)
@@ -65,16 +73,22 @@ class RotaryAttention(Mixer):
 
     def bind(self, tensors):
         names = self._input_names()
-        fused = fuse_rows([tensors[name] for name in names])
+        own = [tensors[name] for name in names]
+        self._carried_at = sum(t.shape[0] for t in own)
+        carried, carried_bias = self._carried or (None, None)
+        fused = fuse_rows(own + ([carried.to(own[0].dtype)] if carried is not None else []))
         self.w_in = kernels.pack_matrix(fused) if fused.is_cuda else fused
         self.b_in = None
-        if self.biases:
+        if self.biases or carried_bias is not None:
             self.b_in = torch.zeros((fused.shape[0],), dtype=torch.float32, device=fused.device)
             at = 0
             for name in names:
                 rows = tensors[name].shape[0]
-                self.b_in[at : at + rows] = tensors[name + ".b"]
+                if self.biases:
+                    self.b_in[at : at + rows] = tensors[name + ".b"]
                 at += rows
+            if carried_bias is not None:
+                self.b_in[at : at + carried.shape[0]] = carried_bias
         o = tensors["o"]
         self.o = kernels.pack_matrix(o.contiguous()) if o.is_cuda else o
         self.o_bias = tensors.get("o.b")
@@ -88,6 +102,8 @@ class RotaryAttention(Mixer):
         if ctx.write_cache != self.own_keys:
             raise ValueError("a layer with keys and values of its own writes its cache layer, and only such a layer does")
         fused = kernels.linear(x, self.w_in, self.b_in, out_dtype=torch.float32)
+        if self._carried is not None:
+            ctx.extra["carried"] = fused[:, self._carried_at : self._carried_at + self._carried[0].shape[0]]
         k_at = self.q_width if self.own_keys else None
         v_at = self.q_width + self.k_width if self.own_keys else None
         rotary, turn = self.rotary, self.value_rotary

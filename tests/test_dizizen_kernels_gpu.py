@@ -51,24 +51,25 @@ def rotate_neighbours(x, positions, dims, base, sign=1.0):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("own_keys", [True, False])
 @pytest.mark.parametrize("pairing", ["half", "neighbours"])
+@pytest.mark.parametrize("lead", [3, 4])   # columns in front of the queries: with 4 the heads start on 16 bytes, and whole fours take the kernel for them
 @pytest.mark.parametrize("dim,vdim,heads,kv_heads,rot_dims,v_dims", [(16, 16, 4, 2, 8, 16), (24, 8, 3, 3, 24, 8), (8, 40, 2, 1, 0, 40), (64, 64, 6, 2, 32, 64),
-                                                                     (10, 6, 3, 1, 4, 6), (128, 192, 2, 1, 128, 192), (20, 12, 5, 5, 6, 4)])
-def test_rows_are_rotated_and_values_are_kept_turned(dtype, own_keys, pairing, dim, vdim, heads, kv_heads, rot_dims, v_dims):
+                                                                     (10, 6, 3, 1, 4, 6), (128, 192, 2, 1, 128, 192), (20, 12, 5, 5, 6, 4), (32, 48, 4, 4, 16, 48)])
+def test_rows_are_rotated_and_values_are_kept_turned(dtype, own_keys, pairing, lead, dim, vdim, heads, kv_heads, rot_dims, v_dims):
     k = kernels()
     rng = np.random.default_rng(dim + vdim)
     rows, page_size, n_pages = 9, 4, 8
     head_size = -(-max(dim, vdim) // 16) * 16
     qw, kw, vw = heads * dim, kv_heads * dim, kv_heads * vdim
-    fused = rng.normal(0, 2, (rows, 3 + qw + kw + vw + 5)).astype(np.float32).astype(np.float64)   # [3 columns of something else | q | k | v | 5 more]
+    fused = rng.normal(0, 2, (rows, lead + qw + kw + vw + 8 - lead)).astype(np.float32).astype(np.float64)   # [columns of something else | q | k | v | more]
     positions = np.array([0, 1, 2, 63, 64, 65, 500, 1100, 7])
     slots = np.array([5, 4, 31, -1, 0, 1, 2, 3, 17])
     base, v_base = 300.0, 40.0
     k_pages = torch.full((n_pages, kv_heads, page_size, head_size), 7.0, dtype=dtype).cuda()
     v_pages = torch.full((n_pages, kv_heads, page_size, head_size), 7.0, dtype=dtype).cuda()
-    q = k.map_rows(gpu(fused), 3, 3 + qw if own_keys else None, 3 + qw + kw if own_keys else None, None, None, 1.0, frequencies(rot_dims, base), rot_dims,
+    q = k.map_rows(gpu(fused), lead, lead + qw if own_keys else None, lead + qw + kw if own_keys else None, None, None, 1.0, frequencies(rot_dims, base), rot_dims,
                    ints(positions), ints(slots), k_pages, v_pages, heads, kv_heads, 1, dim, vdim, v_frequencies=frequencies(v_dims, v_base), v_rot_dims=v_dims,
                    v_pairing=pairing)
-    want_q = plain.rotate_halves(fused[:, 3 : 3 + qw].reshape(rows, heads, dim), positions, rot_dims, base)
+    want_q = plain.rotate_halves(fused[:, lead : lead + qw].reshape(rows, heads, dim), positions, rot_dims, base)
     got_q = q.float().cpu().numpy().reshape(rows, heads, head_size)
     np.testing.assert_allclose(got_q[..., :dim], rounded(want_q, dtype), **tol(dtype))
     assert not got_q[..., dim:].any()
@@ -76,8 +77,8 @@ def test_rows_are_rotated_and_values_are_kept_turned(dtype, own_keys, pairing, d
     if not own_keys:
         assert (kp == 7.0).all() and (vp == 7.0).all()
         return
-    want_k = plain.rotate_halves(fused[:, 3 + qw : 3 + qw + kw].reshape(rows, kv_heads, dim), positions, rot_dims, base)
-    v = fused[:, 3 + qw + kw : 3 + qw + kw + vw].reshape(rows, kv_heads, vdim)
+    want_k = plain.rotate_halves(fused[:, lead + qw : lead + qw + kw].reshape(rows, kv_heads, dim), positions, rot_dims, base)
+    v = fused[:, lead + qw + kw : lead + qw + kw + vw].reshape(rows, kv_heads, vdim)
     want_v = plain.rotate_halves(v, positions, v_dims, v_base) if pairing == "half" else rotate_neighbours(v, positions, v_dims, v_base)
     written = set()
     for row, slot in enumerate(slots):
@@ -96,13 +97,14 @@ def test_rows_are_rotated_and_values_are_kept_turned(dtype, own_keys, pairing, d
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("pairing", ["half", "neighbours"])
-@pytest.mark.parametrize("heads,in_size,out_size,dims", [(4, 16, 16, 16), (3, 48, 36, 36), (2, 64, 40, 8), (5, 32, 12, 0), (2, 192, 192, 192), (1, 16, 6, 6)])
-def test_heads_are_turned_back_by_the_rows_position(dtype, pairing, heads, in_size, out_size, dims):
+@pytest.mark.parametrize("spare", [5, 8])   # columns behind the heads: with 8 the rows lie whole fours apart
+@pytest.mark.parametrize("heads,in_size,out_size,dims", [(4, 16, 16, 16), (3, 48, 36, 36), (2, 64, 40, 8), (5, 32, 12, 0), (2, 192, 192, 192), (1, 16, 6, 6), (6, 64, 64, 64)])
+def test_heads_are_turned_back_by_the_rows_position(dtype, pairing, spare, heads, in_size, out_size, dims):
     k = kernels()
     rng = np.random.default_rng(in_size + out_size)
     rows = 7
     x = rng.normal(0, 1, (rows, heads, in_size)).astype(np.float32).astype(np.float64)
-    wide = np.concatenate([x.reshape(rows, -1), np.zeros((rows, 5))], axis=1)   # rows with something behind the heads: strided
+    wide = np.concatenate([x.reshape(rows, -1), np.zeros((rows, spare))], axis=1)   # rows with something behind the heads: strided
     positions = np.array([0, 1, 63, 64, 999, 1500, 3])
     for sign in (1.0, -1.0):
         got = k.turn_heads(gpu(wide)[:, : heads * in_size], frequencies(dims, 77.0), dims, ints(positions), heads, in_size, out_size, sign=sign, pairing=pairing,
