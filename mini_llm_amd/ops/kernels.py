@@ -272,18 +272,22 @@ def split_blocks(weight, dtype, rows: int = 1) -> int:
     return int(library().mllm_gemm_split_blocks(int(rows), n, k, _code(dtype)))
 
 
-def linear_split(x, weight, k_blocks: int):
+def linear_split(x, weight, k_blocks: int, out=None):
     """x @ weight.T as ``k_blocks`` partial products over consecutive parts of K: float32
     [k_blocks, rows, out]; their sum is the product. The blocks of a product with few output
     columns each read whole rows of x; cut along K they read a part, and many more run. x may be
-    PackedRows (up to 64 rows)."""
+    PackedRows (up to 64 rows). ``out``: float32 [>= k_blocks, rows, out] whose first k_blocks matrices are written (a caller
+    that has one more addend of the same shape keeps it behind them)."""
     x_ptr, x_packed, m, k, x_dtype, device = _rows(x, "x")
     w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x_dtype)
     if not (w_cols == k):
         raise OperandError(f"x has {k} columns but weight has {w_cols}")
-    partials = torch.empty((k_blocks, m, n), dtype=torch.float32, device=device)
-    check(library().mllm_gemm_split(x_ptr, w_ptr, w_packed, _ptr(partials), m, n, k, _code(x_dtype), int(k_blocks), x_packed, _stream()))
-    return partials
+    if out is None:
+        out = torch.empty((k_blocks, m, n), dtype=torch.float32, device=device)
+    _device_tensor(out, "out", torch.float32, 3)
+    _require(out.shape[0] >= k_blocks and tuple(out.shape[1:]) == (m, n), "out does not hold the partial products")
+    check(library().mllm_gemm_split(x_ptr, w_ptr, w_packed, _ptr(out), m, n, k, _code(x_dtype), int(k_blocks), x_packed, _stream()))
+    return out
 
 
 def convert(src, dtype, transpose=False, out=None):
@@ -711,6 +715,20 @@ def _pending(hidden):
         _device_tensor(bias, "the pending bias", torch.float32, 1)
         _require(bias.shape[0] == width, "the pending bias does not match the stream")
     return base, partials, bias, 0 if partials is None else partials.shape[0]
+
+
+@dataclass
+class BranchRows:
+    """A branch's result whose last sums are not taken yet: ``rows`` (float32 [rows, width], or [n, rows, width], the partial products of a
+    product cut along K and whatever else has their shape and joins their sum) plus ``bias`` (float32 [width] or None). Whoever adds the
+    branch to the stream takes the sums on its way in (``branch_join``)."""
+
+    rows: torch.Tensor
+    bias: torch.Tensor | None = None
+
+    @property
+    def shape(self):
+        return self.rows.shape[-2:]
 
 
 @dataclass
@@ -1302,12 +1320,12 @@ def route(logits, n_experts: int, top: int, *, correction=None, n_groups: int = 
     return weights
 
 
-def expert_unit(up, weights, n_routed: int, ff: int, shared: int = 0, *, h=None, n_identity: int = 0):
+def expert_unit(up, weights, n_routed: int, ff: int, shared: int = 0, *, h=None, n_identity: int = 0, carried_out=None):
     """Between the up product over all experts' matrices and the down product over all their down matrices: ``up`` [rows, n_routed * ff +
     shared] -> relu(up)^2 times the row's weight for the unit's expert (``weights``: float32 [rows, >= n_routed + n_identity] as ``route``
     leaves them; the last ``shared`` units belong to an expert every row uses, weight 1). With ``n_identity`` experts that hand their
     input on (``h``: the layer's input rows, of up's type) also returns float32 [rows, width], h times the sum of those experts' weights
-    (else None)."""
+    (else None), written into ``carried_out`` if one is given."""
     _device_tensor(up, "up", dim=2)
     n = up.shape[0]
     _require(up.shape[1] == n_routed * ff + shared, "the hidden units do not match the experts")
@@ -1318,7 +1336,9 @@ def expert_unit(up, weights, n_routed: int, ff: int, shared: int = 0, *, h=None,
         _device_tensor(h, "h", up.dtype, 2)
         _require(h.shape[0] == n, "h and up differ in rows")
         width = h.shape[1]
-        carried = torch.empty((n, width), dtype=torch.float32, device=up.device)
+        carried = torch.empty((n, width), dtype=torch.float32, device=up.device) if carried_out is None else carried_out
+        _device_tensor(carried, "carried_out", torch.float32, 2)
+        _require(tuple(carried.shape) == (n, width), "carried_out has the wrong shape")
     out = torch.empty_like(up)
     check(library().mllm_expert_unit(_ptr(up), _ptr(out), _ptr(weights), weights.stride(0), n, int(n_routed), int(ff), int(shared), _ptr(h if n_identity else None),
                                      _ptr(carried), int(n_identity), int(width), _code(up.dtype), _stream()))
@@ -1329,11 +1349,17 @@ def branch_join(stream, a, b=None, *, a_bias=None, b_bias=None, scale_a=None, sc
                 mult: float = 1.0, next_weight=None, one_plus: bool = False, eps: float = 0.0, out_dtype=None):
     """stream + mult * (scale_a * sigmoid(gate_a) * a + scale_b * sigmoid(gate_b) * b), float32 [rows, width]: the sum of a layer whose
     branches a and b (None: one branch) read the same normed input. a, b: float32 [rows, width] or [n, rows, width], the partial products of
-    a product cut along K, added up here (with ``*_bias``, float32 [width]). ``scale_*``: float32 [width] or None; ``gates``: float32 rows
+    a product cut along K, added up here (with ``*_bias``, float32 [width]), or ``BranchRows`` holding both. ``scale_*``: float32 [width] or None; ``gates``: float32 rows
     (strided) holding a's gate at column ``gate_a_at`` and b's at ``gate_b_at``, before their sigmoid, or None. With ``next_weight`` (and
     ``eps``, ``one_plus``, ``out_dtype``) also returns the sum RMS-normed with that gain, in ``out_dtype``: (sum, normed rows)."""
     _device_tensor(stream, "stream", torch.float32, 2)
     n, width = stream.shape
+    if isinstance(a, BranchRows):
+        _require(a_bias is None, "a brings its own bias")
+        a, a_bias = a.rows, a.bias
+    if isinstance(b, BranchRows):
+        _require(b_bias is None, "b brings its own bias")
+        b, b_bias = b.rows, b.bias
 
     def partials(t, name):
         if t is None:

@@ -163,6 +163,9 @@ class ParallelBlock(Block):
         self._names = names
         self._following = None
         self.scale_1 = self.scale_2 = self.gates = self.gates_bias = None
+        for part in (mixer, feed_forward):   # the sum's kernel takes a branch's bias and the partial products of its last product
+            if part is not None and hasattr(part, "sums_later"):
+                part.sums_later = True
 
     def children(self):
         parts = dict(zip(self._names, (self.norm_1, self.mixer, self.feed_forward)))

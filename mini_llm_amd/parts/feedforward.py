@@ -89,6 +89,7 @@ class ClampedGatedMLP(FeedForward):
         self._names = names
         self.gate_up = self.gate_up_bias = self.down = self.down_bias = None
         self._down_product = BranchProduct()
+        self.sums_later = False   # True: a call without a residual may return kernels.BranchRows (the block that adds the branch takes its sums)
 
     def tensor_specs(self):
         from ..weights.spec import MATRIX, TABLE, VECTOR, Normal, TensorSpec
@@ -114,6 +115,8 @@ class ClampedGatedMLP(FeedForward):
 
     def forward(self, x, residual):
         inner = kernels.gate_unit(kernels.linear(x, self.gate_up, self.gate_up_bias), self.limit, self.alpha, self.shift)
+        if residual is None and self.sums_later:
+            return self._down_product.later(inner, self.down, self.down_bias)
         return self._down_product(inner, self.down, residual, bias=self.down_bias)
 
 

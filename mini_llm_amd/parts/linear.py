@@ -69,18 +69,42 @@ class BranchProduct:
     def __init__(self):
         self._split_blocks = {}
 
+    def blocks(self, x, weight) -> int:
+        """Into how many partial products the product of these rows is cut (1: it stays whole)."""
+        rows = x.shape[0]
+        if rows <= self.FEW_ROWS:
+            return 1
+        bucket = 0 if rows <= 64 else -(-rows // 128)   # the answer is the same inside a bucket
+        k_blocks = self._split_blocks.get((bucket, x.dtype))
+        if k_blocks is None:
+            k_blocks = self._split_blocks[bucket, x.dtype] = kernels.split_blocks(weight, x.dtype, rows)
+        return k_blocks
+
     def __call__(self, x, weight, residual=None, bias=None):
         import torch
 
-        if residual is None and bias is None and x.shape[0] > self.FEW_ROWS:
-            rows = x.shape[0]
-            bucket = 0 if rows <= 64 else -(-rows // 128)   # the answer is the same inside a bucket
-            k_blocks = self._split_blocks.get((bucket, x.dtype))
-            if k_blocks is None:
-                k_blocks = self._split_blocks[bucket, x.dtype] = kernels.split_blocks(weight, x.dtype, rows)
+        if residual is None and bias is None:
+            k_blocks = self.blocks(x, weight)
             if k_blocks > 1:
                 return kernels.linear_split(x, weight, k_blocks)
         return kernels.linear(x, weight, bias, residual=residual, out_dtype=torch.float32)
+
+    def later(self, x, weight, bias=None, spare: int = 0):
+        """For a branch whose sum with the stream is taken by a kernel that also takes a bias and partial products
+        (``kernels.branch_join``): ``kernels.BranchRows`` of the product, cut along K where that pays, and the bias, not yet added. ``spare``:
+        so many more matrices of the product's shape are kept behind the partial products for the caller to fill (they join the sum)."""
+        import torch
+
+        k_blocks = self.blocks(x, weight)
+        if k_blocks == 1 and not spare:
+            return kernels.BranchRows(kernels.linear(x, weight, out_dtype=torch.float32), bias)
+        out = torch.empty((k_blocks + spare, x.shape[0], weight.rows if isinstance(weight, kernels.PackedMatrix) else weight.shape[0]),
+                          dtype=torch.float32, device=x.device if hasattr(x, "device") else x.data.device)
+        if k_blocks == 1:
+            kernels.linear(x, weight, out_dtype=torch.float32, out=out[0])
+        else:
+            kernels.linear_split(x, weight, k_blocks, out=out)
+        return kernels.BranchRows(out, bias)
 
 
 def fuse_rows(matrices, multiple: int = 16):

@@ -49,6 +49,7 @@ class RotaryAttention(Mixer):
         self.q_width, self.k_width, self.v_width, self.o_width = n_heads * dim, n_kv_heads * dim, n_kv_heads * vdim, n_heads * vdim
         self.w_in = self.b_in = self.o = self.o_bias = None
         self._out_product = BranchProduct()
+        self.sums_later = False   # True: a call without a residual may return kernels.BranchRows (the block that adds the branch takes its sums)
         self._carried = None      # (matrix, bias) of rows that ride along in the input product, and where their columns start
         self._carried_at = 0
 
@@ -122,6 +123,8 @@ class RotaryAttention(Mixer):
         if reshape:
             mixed = kernels.turn_heads(mixed, turn.frequencies64(x.device) if turn_dims else None, turn_dims, batch.positions, self.n_heads,
                                        self.head_size, self.vdim, sign=-1.0, pairing="half" if turn is None else turn.pairing, out_dtype=x.dtype)
+        if residual is None and self.sums_later:
+            return self._out_product.later(mixed, self.o, self.o_bias)
         return self._out_product(mixed, self.o, residual, bias=self.o_bias)
 
 

@@ -41,6 +41,7 @@ class RoutedExperts(FeedForward):
         self.router = self.correction = self.up = self.down = None
         self.shared_units = 0   # the shared expert's hidden units and the zeros that fill the up matrix to whole blocks
         self._down_product = BranchProduct()
+        self.sums_later = False   # True: a call without a residual may return kernels.BranchRows (the block that adds the branch takes its sums)
 
     def tensor_specs(self):
         specs = {"router": TensorSpec((self.n_outputs, self.width), TABLE, Normal(self.width ** -0.5))}
@@ -77,6 +78,19 @@ class RoutedExperts(FeedForward):
         weights = kernels.route(logits, self.n_outputs, self.top, correction=self.correction, n_groups=self.n_groups, keep=self.keep, floor=self.floor)
         if self.up is None:   # nothing but experts that hand their input on
             raise ValueError("a routed feed-forward needs at least one expert with matrices")
+        if residual is None and self.sums_later:
+            # the share of the experts that hand h on lies behind the down product's partial products and joins their sum
+            spare = 1 if self.n_identity else 0
+            hidden = kernels.linear(x, self.up)
+            k_blocks = self._down_product.blocks(hidden, self.down)
+            out = torch.empty((k_blocks + spare, hidden.shape[0], self.width), dtype=torch.float32, device=hidden.device)
+            units, _ = kernels.expert_unit(hidden, weights, self.n_experts, self.ff, self.shared_units, h=x, n_identity=self.n_identity,
+                                           carried_out=out[k_blocks] if spare else None)
+            if k_blocks == 1:
+                kernels.linear(units, self.down, out_dtype=torch.float32, out=out[0])
+            else:
+                kernels.linear_split(units, self.down, k_blocks, out=out)
+            return kernels.BranchRows(out, None)
         units, carried = kernels.expert_unit(kernels.linear(x, self.up), weights, self.n_experts, self.ff, self.shared_units, h=x, n_identity=self.n_identity)
         if carried is not None and residual is not None:
             carried = kernels.add(carried, residual)

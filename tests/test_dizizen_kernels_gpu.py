@@ -195,6 +195,11 @@ def test_routed_experts_against_the_plain_sum_over_the_picked(dtype, rows, case)
     stream = np.random.default_rng(1).normal(0, 1, (rows, width)).astype(np.float32)
     with_stream = part.forward(gpu(h, dtype), gpu(stream)).cpu().numpy()
     np.testing.assert_allclose(with_stream, got + stream, atol=1e-4 * max(scale, 1.0), rtol=0)
+    # for a block that takes the sums itself: the partial products of the down product, and the share of the experts that hand h on behind them
+    part.sums_later = True
+    later = part.forward(gpu(h, dtype), None)
+    assert later.bias is None and later.rows.dim() == 3 and later.rows.shape[0] >= (2 if mlp["router"].get("identity") else 1)
+    np.testing.assert_allclose(later.rows.cpu().numpy().astype(np.float64).sum(axis=0), got, atol=1e-4 * max(scale, 1.0), rtol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -243,6 +248,11 @@ def test_the_clamped_gated_feed_forward_part(dtype, rows):
     want = plain.dense_feed_forward(h, {"kind": "dense", "ff": inner, "limit": limit}, tensors, "m.", rnd)
     got = part.forward(gpu(h, dtype), None).cpu().numpy()
     np.testing.assert_allclose(got, want, atol=(3e-5 if dtype == torch.float32 else 3e-2) * np.abs(want).max(), rtol=0)
+    part.sums_later = True   # for a block that takes the sums itself
+    later = part.forward(gpu(h, dtype), None)
+    total = later.rows.cpu().numpy().astype(np.float64)
+    total = (total.sum(axis=0) if total.ndim == 3 else total) + later.bias.cpu().numpy()
+    np.testing.assert_allclose(total, got, atol=1e-4 * np.abs(want).max(), rtol=0)
 
 
 def k_pack(matrix):
