@@ -80,7 +80,7 @@ __global__ __launch_bounds__(64 * JOIN_WAVES) void branch_join_rows_kernel(
         }
         return out;
     };
-    Piece sums[CHUNKS];
+    Piece sums[CHUNKS], gains[CHUNKS];
     float squares = 0.0f;
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
@@ -89,6 +89,7 @@ __global__ __launch_bounds__(64 * JOIN_WAVES) void branch_join_rows_kernel(
         const Piece xs = piece(x + at + d), ga = piece(gate_row + gate_a_at + d), gb = piece(gate_row + gate_b_at + d);
         const Piece sa = piece(scale_a + d), sb = piece(scale_b + d), ba = piece(a_bias + d), bb = piece(b_bias + d);
         Piece first = piece(a + at + d), second = piece(b + at + d);
+        gains[c] = piece(next_weight + d);   // asked for with everything else: the norm behind the sum then waits for no trip of its own
         for (int p = 1; p < n_a; p++) {
             const Piece more = piece(a + (size_t)p * a_stride + at + d);
 #pragma unroll
@@ -122,9 +123,8 @@ __global__ __launch_bounds__(64 * JOIN_WAVES) void branch_join_rows_kernel(
     for (int c = 0; c < CHUNKS; c++) {
         const int d = (c * WAVE + lane) * VEC;
         if (d > last) continue;
-        const Piece gain = piece(next_weight + d);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) rows_out[at + d + e] = from_float<T>(sums[c].v[e] * factor * (one_plus ? 1.0f + gain.v[e] : gain.v[e]));
+        for (int e = 0; e < VEC; e++) rows_out[at + d + e] = from_float<T>(sums[c].v[e] * factor * (one_plus ? 1.0f + gains[c].v[e] : gains[c].v[e]));
     }
 }
 
