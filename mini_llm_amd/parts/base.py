@@ -122,9 +122,9 @@ class Mixer(Part):
     decode_reaches: tuple = ()
 
     # True if the mixer's first product reads the layer's input rows as they are and can carry other output rows along in it:
-    # ``carry_rows(matrix, bias)`` (before the tensors are bound) lays ``matrix`` [n, width] (and its float32 bias, or None) behind the
-    # mixer's own, and every ``forward`` leaves the carried columns, float32 [rows, n], in ``ctx.extra["carried"]``. A block whose
-    # gates read the same rows as its mixer saves a product this way.
+    # ``carry_rows(name, matrix, bias)`` (before the tensors are bound) lays ``matrix`` [n, width] (and its float32 bias, or None) behind the
+    # mixer's own, and every ``forward`` leaves the carried columns, float32 [rows, n], in ``ctx.extra["carried"][name]``. A block whose
+    # gates, or whose feed-forward's router, read the same rows as its mixer saves a product this way.
     carries_rows = False
 
     def kv_need(self) -> KVNeed | None:

@@ -162,6 +162,7 @@ class ParallelBlock(Block):
         self.width, self.compute_dtype, self.mult, self.layer_scale, self.gated = width, compute_dtype, float(mult), bool(layer_scale), bool(gated)
         self._names = names
         self._following = None
+        self._feed_forward_rides = False
         self.scale_1 = self.scale_2 = self.gates = self.gates_bias = None
         for part in (mixer, feed_forward):   # the sum's kernel takes a branch's bias and the partial products of its last product
             if part is not None and hasattr(part, "sums_later"):
@@ -205,11 +206,35 @@ class ParallelBlock(Block):
             self.gates_bias = torch.zeros((fused.shape[0],), dtype=torch.float32, device=fused.device)
             for index, n in enumerate(self._branches()):
                 self.gates_bias[index * self.width : (index + 1) * self.width] = tensors["rg" + n + ".b"]
-            if self.mixer.carries_rows:   # the gates ride along in the mixer's own first product (this part is bound before its children)
-                self.mixer.carry_rows(fused, self.gates_bias)
+            if self.mixer.carries_rows:   # the gates ride along in the mixer's own first product (the mixer is bound after this part)
+                self.mixer.carry_rows("gates", fused, self.gates_bias)
                 self.gates = None
             else:
                 self.gates = kernels.pack_matrix(fused) if fused.is_cuda else fused
+        self._ride_feed_forward()
+
+    def _ride_feed_forward(self):
+        """A feed-forward whose first small product reads the layer's input rows (a router) sends it along in the mixer's too."""
+        rider = getattr(self.feed_forward, "rows_to_carry", None)
+        self._feed_forward_rides = False
+        if rider is not None and self.mixer.carries_rows:
+            rows = rider()
+            if rows is not None:
+                self.mixer.carry_rows("feed_forward", *rows)
+                self._feed_forward_rides = True
+
+    def bind_named(self, tensors: dict, prefix: str = "") -> None:
+        # the feed-forward first, this part's own tensors next, the mixer last: both may hand rows to the mixer, which lays them behind its
+        # own when it is bound
+        if self.feed_forward is not None:
+            self.feed_forward.bind_named(tensors, prefix + self._names[2])
+        own = {name: tensors[prefix + name] for name in self.tensor_specs()}
+        if own:
+            self.bind(own)
+        else:
+            self._ride_feed_forward()
+        self.norm_1.bind_named(tensors, prefix + self._names[0])
+        self.mixer.bind_named(tensors, prefix + self._names[1])
 
     def forward(self, hidden, ctx: LayerContext):
         import torch
@@ -223,9 +248,12 @@ class ParallelBlock(Block):
             rows = self.norm_1.forward(stream, self.compute_dtype)
         gates = kernels.linear(rows, self.gates, self.gates_bias, out_dtype=torch.float32) if self.gated and self.gates is not None else None
         first = self.mixer.forward(rows, None, ctx)
+        carried = ctx.extra.pop("carried", {})
         if self.gated and self.gates is None:
-            gates = ctx.extra.pop("carried")
-        second = self.feed_forward.forward(rows, None) if self.feed_forward is not None else None
+            gates = carried["gates"]
+        second = None
+        if self.feed_forward is not None:
+            second = self.feed_forward.forward(rows, None, carried=carried["feed_forward"]) if self._feed_forward_rides else self.feed_forward.forward(rows, None)
         following = self._following
         ahead = {}
         if following is not None and hasattr(following, "one_plus") and getattr(following, "out_scale", 1.0) == 1.0:

@@ -50,13 +50,13 @@ class RotaryAttention(Mixer):
         self.w_in = self.b_in = self.o = self.o_bias = None
         self._out_product = BranchProduct()
         self.sums_later = False   # True: a call without a residual may return kernels.BranchRows (the block that adds the branch takes its sums)
-        self._carried = None      # (matrix, bias) of rows that ride along in the input product, and where their columns start
-        self._carried_at = 0
+        self._carried = {}        # name -> (matrix, bias) of rows that ride along in the input product
+        self._carried_at = {}     # name -> (first column, columns) in the product's rows
 
-    def carry_rows(self, matrix, bias=None):
+    def carry_rows(self, name, matrix, bias=None):
         if matrix.dim() != 2 or matrix.shape[1] != self.width:
             raise ValueError(f"rows that ride along read the same {self.width} inputs")
-        self._carried = (matrix, bias)
+        self._carried[name] = (matrix, bias)
 
     def _input_names(self):
         return ("q", "k", "v") if self.own_keys else ("q",)
@@ -75,12 +75,15 @@ class RotaryAttention(Mixer):
     def bind(self, tensors):
         names = self._input_names()
         own = [tensors[name] for name in names]
-        self._carried_at = sum(t.shape[0] for t in own)
-        carried, carried_bias = self._carried or (None, None)
-        fused = fuse_rows(own + ([carried.to(own[0].dtype)] if carried is not None else []))
+        at = sum(t.shape[0] for t in own)
+        self._carried_at = {}
+        for rider, (matrix, _) in self._carried.items():
+            self._carried_at[rider] = (at, matrix.shape[0])
+            at += matrix.shape[0]
+        fused = fuse_rows(own + [matrix.to(own[0].dtype) for matrix, _ in self._carried.values()])
         self.w_in = kernels.pack_matrix(fused) if fused.is_cuda else fused
         self.b_in = None
-        if self.biases or carried_bias is not None:
+        if self.biases or any(bias is not None for _, bias in self._carried.values()):
             self.b_in = torch.zeros((fused.shape[0],), dtype=torch.float32, device=fused.device)
             at = 0
             for name in names:
@@ -88,8 +91,10 @@ class RotaryAttention(Mixer):
                 if self.biases:
                     self.b_in[at : at + rows] = tensors[name + ".b"]
                 at += rows
-            if carried_bias is not None:
-                self.b_in[at : at + carried.shape[0]] = carried_bias
+            for rider, (_, bias) in self._carried.items():
+                if bias is not None:
+                    first, n = self._carried_at[rider]
+                    self.b_in[first : first + n] = bias
         o = tensors["o"]
         self.o = kernels.pack_matrix(o.contiguous()) if o.is_cuda else o
         self.o_bias = tensors.get("o.b")
@@ -103,8 +108,8 @@ class RotaryAttention(Mixer):
         if ctx.write_cache != self.own_keys:
             raise ValueError("a layer with keys and values of its own writes its cache layer, and only such a layer does")
         fused = kernels.linear(x, self.w_in, self.b_in, out_dtype=torch.float32)
-        if self._carried is not None:
-            ctx.extra["carried"] = fused[:, self._carried_at : self._carried_at + self._carried[0].shape[0]]
+        if self._carried_at:
+            ctx.extra["carried"] = {rider: fused[:, first : first + n] for rider, (first, n) in self._carried_at.items()}
         k_at = self.q_width if self.own_keys else None
         v_at = self.q_width + self.k_width if self.own_keys else None
         rotary, turn = self.rotary, self.value_rotary

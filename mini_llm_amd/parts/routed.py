@@ -38,7 +38,7 @@ class RoutedExperts(FeedForward):
         self.width, self.n_experts, self.ff, self.top, self.n_identity = width, n_experts, ff, top, n_identity
         self.n_groups, self.keep, self.has_correction, self.shared_ff, self.floor = n_groups, keep, bool(correction), shared_ff or 0, float(floor)
         self.n_outputs = total
-        self.router = self.correction = self.up = self.down = None
+        self.router = self.correction = self.up = self.down = self._router_rows = None
         self.shared_units = 0   # the shared expert's hidden units and the zeros that fill the up matrix to whole blocks
         self._down_product = BranchProduct()
         self.sums_later = False   # True: a call without a residual may return kernels.BranchRows (the block that adds the branch takes its sums)
@@ -60,6 +60,7 @@ class RoutedExperts(FeedForward):
     def bind(self, tensors):
         names = [f"e{e}." for e in range(self.n_experts)] + (["shared."] if self.shared_ff else [])
         router = fuse_rows([tensors["router"]])
+        self._router_rows = router
         self.router = kernels.pack_matrix(router) if router.is_cuda else router
         self.correction = tensors.get("correction")
         up = fuse_rows([tensors[name + "up"] for name in names]) if names else None
@@ -73,8 +74,13 @@ class RoutedExperts(FeedForward):
         down = down.contiguous()
         self.up, self.down = (kernels.pack_matrix(up), kernels.pack_matrix(down)) if up.is_cuda else (up, down)
 
-    def forward(self, x, residual):
-        logits = kernels.linear(x, self.router, out_dtype=torch.float32)
+    def rows_to_carry(self):
+        """The router's matrix (and no bias), for a block that lets another product over the same input rows carry it along; ``forward`` is
+        then given the router's sums as ``carried``."""
+        return self._router_rows, None
+
+    def forward(self, x, residual, carried=None):
+        logits = carried if carried is not None else kernels.linear(x, self.router, out_dtype=torch.float32)
         weights = kernels.route(logits, self.n_outputs, self.top, correction=self.correction, n_groups=self.n_groups, keep=self.keep, floor=self.floor)
         if self.up is None:   # nothing but experts that hand their input on
             raise ValueError("a routed feed-forward needs at least one expert with matrices")
