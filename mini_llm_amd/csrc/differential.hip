@@ -54,6 +54,35 @@ __global__ __launch_bounds__(64 * MAP_WAVES) void turn_heads_kernel(const float*
         to[d] = from_float<T>(d < rot_dims ? turned_element(from, d, rot_dims, neighbours, position, frequencies, sign) : from[d]);
 }
 
+// Four neighbouring elements out, in 32-bit or rounded to bfloat16.
+template <typename T>
+__device__ __forceinline__ void store_four(T* to, f32x4 made) {
+    if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<f32x4*>(to) = made;
+    } else {
+        bf16x4 narrow;
+#pragma unroll
+        for (int e = 0; e < 4; e++) narrow[e] = from_float<T>(made[e]);
+        *reinterpret_cast<bf16x4*>(to) = narrow;
+    }
+}
+
+// Four pairs (from[d + e], from[d + half + e]) turned by sign x position x frequencies[d + e] and stored at to + d and to + d + half: the
+// sine and cosine of a pair are taken once for both its elements.
+template <typename T>
+__device__ __forceinline__ void turn_four_pairs(const float* from, T* to, int d, int half, int position, const double* frequencies, float sign) {
+    const f32x4 firsts = *reinterpret_cast<const f32x4*>(from + d), seconds = *reinterpret_cast<const f32x4*>(from + d + half);
+    f32x4 a, b;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float x, y;
+        turned(firsts[e], seconds[e], position, sign * frequencies[d + e], x, y);
+        a[e] = x, b[e] = y;
+    }
+    store_four(to + d, a);
+    store_four(to + d + half, b);
+}
+
 // turn_heads_kernel four neighbouring elements a thread (pairing of halves; turned elements, heads and strides in whole fours, rows on 16 bytes).
 template <typename T>
 __global__ __launch_bounds__(256) void turn_heads_pieces_kernel(const float* __restrict__ in, int in_stride, T* __restrict__ out, int out_stride,
@@ -65,30 +94,12 @@ __global__ __launch_bounds__(256) void turn_heads_pieces_kernel(const float* __r
     const int row = (int)(index / (n_heads * quads)), within = (int)(index % (n_heads * quads));
     const int head = within / quads, d = (within % quads) * 4;
     const float* from = in + (size_t)row * in_stride + (size_t)head * in_size;
-    f32x4 made = *reinterpret_cast<const f32x4*>(from + d);
-    if (d < rot_dims) {
-        const int half = rot_dims / 2;
-        const bool first = d < half;
-        const int pair = first ? d : d - half;
-        const f32x4 partner = *reinterpret_cast<const f32x4*>(from + (first ? d + half : d - half));
-        const int position = positions[row];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            float a, b;
-            if (first) turned(made[e], partner[e], position, sign * frequencies[pair + e], a, b);
-            else turned(partner[e], made[e], position, sign * frequencies[pair + e], b, a);
-            made[e] = a;
-        }
+    T* to = out + (size_t)row * out_stride + (size_t)head * out_size;
+    if (d < rot_dims) {   // the thread of a pair's first element makes both; the thread of the second has nothing to do
+        if (d < rot_dims / 2) turn_four_pairs(from, to, d, rot_dims / 2, positions[row], frequencies, sign);
+        return;
     }
-    T* to = out + (size_t)row * out_stride + (size_t)head * out_size + d;
-    if constexpr (sizeof(T) == 4) {
-        *reinterpret_cast<f32x4*>(to) = made;
-    } else {
-        bf16x4 narrow;
-#pragma unroll
-        for (int e = 0; e < 4; e++) narrow[e] = from_float<T>(made[e]);
-        *reinterpret_cast<bf16x4*>(to) = narrow;
-    }
+    store_four(to + d, *reinterpret_cast<const f32x4*>(from + d));
 }
 
 // A wave per (row, item); a row's items are its n_heads * maps queries, then (where the layer keeps keys and values of its own: k_at
@@ -208,32 +219,13 @@ __global__ __launch_bounds__(256) void rotate_rows_pieces_kernel(
             size = vdim, turned_dims = v_frequencies ? v_rot_dims : 0, f = v_frequencies;
         }
     }
+    if (d < turned_dims) {   // the thread of a pair's first element makes both; the thread of the second has nothing to do
+        if (d < turned_dims / 2) turn_four_pairs(in, out, d, turned_dims / 2, positions[row], f, 1.0f);
+        return;
+    }
     f32x4 made = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (d < size) {
-        made = *reinterpret_cast<const f32x4*>(in + d);
-        if (d < turned_dims) {
-            const int half = turned_dims / 2;
-            const bool first = d < half;
-            const int pair = first ? d : d - half;
-            const f32x4 partner = *reinterpret_cast<const f32x4*>(in + (first ? d + half : d - half));
-            const int position = positions[row];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                float a, b;
-                if (first) turned(made[e], partner[e], position, f[pair + e], a, b);
-                else turned(partner[e], made[e], position, f[pair + e], b, a);
-                made[e] = a;
-            }
-        }
-    }
-    if constexpr (sizeof(T) == 4) {
-        *reinterpret_cast<f32x4*>(out + d) = made;
-    } else {
-        bf16x4 narrow;
-#pragma unroll
-        for (int e = 0; e < 4; e++) narrow[e] = from_float<T>(made[e]);
-        *reinterpret_cast<bf16x4*>(out + d) = narrow;
-    }
+    if (d < size) made = *reinterpret_cast<const f32x4*>(in + d);
+    store_four(out + d, made);
 }
 
 // A wave per (row, head): with a1 and a2 the results of the head's two maps (attention heads (g * 2 + 0) * R + r and (g * 2 + 1) * R + r
