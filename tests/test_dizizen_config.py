@@ -182,3 +182,38 @@ def test_greedy_generation_is_prefix_stable():
     w = plain.as_float64(plain.random_weights(raw, 6))
     new = plain.greedy(raw, w, [3, 1, 4], 5)
     assert plain.greedy(raw, w, [3, 1, 4] + new[:2], 3) == new[2:]
+
+
+def test_the_gates_and_the_router_ride_in_the_attention_input_product():
+    # bound on the host (nothing runs there): the attention's fused input matrix holds q, k, v, then the block's two gate matrices, then
+    # the router's rows, and the biases lie beside their rows
+    import torch
+
+    from mini_llm_amd.weights import bind_tensors
+
+    raw = CASES["mixed"]
+    built = build_model(config_from_dict(raw), "float32")
+    weights = plain.random_weights(raw, 11)
+    bind_tensors(built, {name: torch.tensor(value) for name, value in weights.items()}, "cpu")
+    width = raw["width"]
+    for index, (block, entry) in enumerate(zip(built.blocks, raw["layers"])):
+        mixer, m = block.mixer, entry["mixer"]
+        own = m["heads"] * m["dim"] + (0 if "kv_from" in m else m["kv_heads"] * (m["dim"] + m["vdim"]))
+        gates_at, gates_n = mixer._carried_at["gates"]
+        assert gates_at == own and gates_n >= (2 if entry["mlp"] else 1) * width and block.gates is None
+        fused, bias = mixer.w_in.numpy(), mixer.b_in.numpy()
+        np.testing.assert_array_equal(fused[: m["heads"] * m["dim"]], weights[f"l{index}.mix.q"])
+        np.testing.assert_array_equal(fused[gates_at : gates_at + width], weights[f"l{index}.rg1"])
+        np.testing.assert_array_equal(bias[gates_at : gates_at + width], weights[f"l{index}.rg1.b"])
+        np.testing.assert_array_equal(bias[: m["heads"] * m["dim"]], weights[f"l{index}.mix.q.b"])
+        if entry["mlp"]:
+            np.testing.assert_array_equal(fused[gates_at + width : gates_at + 2 * width], weights[f"l{index}.rg2"])
+            np.testing.assert_array_equal(bias[gates_at + width : gates_at + 2 * width], weights[f"l{index}.rg2.b"])
+        routed = (entry["mlp"] or {}).get("kind") == "moe"
+        assert ("feed_forward" in mixer._carried_at) == routed == block._feed_forward_rides
+        if routed:
+            at, n = mixer._carried_at["feed_forward"]
+            outputs = weights[f"l{index}.mlp.router"].shape[0]
+            assert at == gates_at + gates_n and n >= outputs
+            np.testing.assert_array_equal(fused[at : at + outputs], weights[f"l{index}.mlp.router"])
+            assert not bias[at : at + n].any() and not fused[at + outputs : at + n].any()
